@@ -1,0 +1,73 @@
+/* C ABI of the routed-expert MXFP8 FFN forward (the "MoK" hot path) on gfx950.
+ *
+ * What the reference reaches through MoKHost.forward -> HostSession.launch
+ * (campaigns/mok/host/mok_port_host.py:185-205, pipec/src/pipec2/host/broker.py:741-751)
+ * with the residues its owner providers build
+ * (campaigns/mok/port/gemm/provider.cu:217-303, campaigns/mok/port/act_gptoss/provider.cu),
+ * is reached here through plk_mok_session_create + plk_mok_forward: the session owns one
+ * loaded pipeline image (linked or one-unit build) and its device-resident params images;
+ * forward fills the framework / GEMM / activation params and launches the gate-up pass
+ * and the down pass on the caller's stream.  All tensor arguments are device addresses
+ * owned by the caller; nothing is allocated per call.
+ *
+ * Operand layouts (all row-major):
+ *   x_q [T,H] e4m3, x_sc [T,ld_sc_h] e8m0 (one byte per 32 elements of H; ld_sc_h % 4 == 0)
+ *   w_gate_q / w_up_q [E,I,H], scales [E,I,ld_sc_h];  w_down_q [E,H,I], scales [E,H,ld_sc_i]
+ *   tokens_per_expert [E] i32, row_token [R] i32 (routed row -> token; 0 = rows are tokens)
+ *   hidden_q [R,I] e4m3 + hidden_sc [R,ld_sc_i] (written by pass 1, read by pass 2)
+ *   y [R,H] bf16 */
+#ifndef PLK_MOK_H
+#define PLK_MOK_H
+
+#include "plk_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* what link.json says about the image (pipec link output: params.entries, threads, dyn_smem_bytes) */
+typedef struct plk_mok_link_info {
+  uint32_t struct_bytes;       /* sizeof(plk_mok_link_info) */
+  uint32_t params_bytes;       /* total size of the params image */
+  uint32_t framework_offset;   /* offset of MokFrameworkParams in the image */
+  uint32_t gemm_offset;        /* offset of MokGemmResidue */
+  uint32_t act_offset;         /* offset of MokActResidue */
+  uint32_t threads;            /* workgroup size */
+  uint32_t dyn_lds_bytes;      /* dynamic LDS per workgroup */
+  uint32_t workgroups_per_cu;  /* occupancy the image was solved for */
+} plk_mok_link_info;
+
+typedef struct plk_mok_problem {
+  uint32_t struct_bytes; /* sizeof(plk_mok_problem) */
+  int32_t num_tokens;    /* T */
+  int32_t hidden;        /* H = d_model */
+  int32_t intermediate;  /* I = d_ff */
+  int32_t num_experts;   /* E */
+  int32_t routed_rows;   /* R = sum(tokens_per_expert) */
+  int32_t ld_sc_h;       /* scale row pitch for K = H operands */
+  int32_t ld_sc_i;       /* scale row pitch for K = I operands */
+  float swiglu_limit;
+  int32_t reserved;
+  uint64_t x_q, x_sc, row_token, tokens_per_expert;
+  uint64_t w_gate_q, w_gate_sc, w_up_q, w_up_sc, w_down_q, w_down_sc;
+  uint64_t hidden_q, hidden_sc, y;
+} plk_mok_problem;
+
+typedef struct plk_mok_session plk_mok_session;
+
+int plk_mok_session_create(const void* image, size_t image_bytes, const plk_mok_link_info* link, plk_mok_session** out);
+int plk_mok_session_destroy(plk_mok_session* s);
+/* both passes; or one of them (pass 1 = gate/up + SwiGLU + requant, pass 2 = down) */
+int plk_mok_forward(plk_mok_session* s, const plk_mok_problem* p, void* stream);
+int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass, void* stream);
+
+/* MXFP8 block quantiser on the device (what ops.mxfp8_quantize does for the reference's
+ * harness, campaigns/mok/host/mok_port_host.py:122): src is fp32 (src_is_bf16 = 0) or bf16
+ * [rows, k], dst_q [rows, k] e4m3, dst_sc [rows, ld_sc] e8m0 (padding bytes zeroed). */
+int plk_mxfp8_quantize(uint64_t src, int src_is_bf16, int64_t rows, int32_t k, uint64_t dst_q, uint64_t dst_sc,
+                       int32_t ld_sc, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,239 @@
+// Implementation of include/plk_mok.h: host side of the routed-expert MXFP8 FFN forward.
+// Builds the params image the linked pipeline kernel reads (framework schedule params,
+// GEMM residue, activation residue at their linked offsets), keeps it resident on the
+// device, and launches the gate/up pass and the down pass.
+#include "plk_mok.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <vector>
+
+#include "../stages/mok/include/mok_abi.h"
+
+extern "C" int plk_hip_set_error(int code, const char* what);
+
+namespace {
+constexpr int TILE_X = 128;  // routed rows per workgroup tile   (fact mok.gemm.TILE_X)
+constexpr int TILE_W = 256;  // weight rows per workgroup tile   (fact mok.gemm.TILE_W)
+constexpr int K_STEP = 64;
+constexpr int MAX_EXPERTS = 256;
+constexpr int NUM_XCD = 8;
+}  // namespace
+
+struct plk_mok_session {
+  plk_hip_module* module = nullptr;
+  plk_hip_function* kernel = nullptr;
+  plk_mok_link_info link{};
+  uint64_t params_dev[2] = {0, 0};            // device copies of the two passes' params images
+  std::vector<unsigned char> params_host[2];  // what the device copies hold
+  int32_t compute_units = 0;
+};
+
+static int check_problem(const plk_mok_problem* p) {
+  if (!p || p->struct_bytes != sizeof(plk_mok_problem))
+    return plk_hip_set_error(PLK_E_VERSION, "plk_mok: problem struct size mismatch");
+  if (p->num_experts <= 0 || p->num_experts > MAX_EXPERTS)
+    return plk_hip_set_error(PLK_E_CAPACITY, "plk_mok: num_experts must be in 1..256");
+  if (p->hidden <= 0 || p->intermediate <= 0 || p->hidden % K_STEP || p->intermediate % K_STEP)
+    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: hidden and intermediate must be positive multiples of 64");
+  if (p->ld_sc_h % 4 || p->ld_sc_i % 4 || p->ld_sc_h * 32 < p->hidden || p->ld_sc_i * 32 < p->intermediate)
+    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: scale pitch must be a multiple of 4 covering K/32 blocks");
+  if (p->num_tokens < 0 || p->routed_rows < 0)
+    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: negative row count");
+  if (p->routed_rows && (!p->x_q || !p->x_sc || !p->tokens_per_expert || !p->w_gate_q || !p->w_gate_sc ||
+                         !p->w_up_q || !p->w_up_sc || !p->w_down_q || !p->w_down_sc || !p->hidden_q ||
+                         !p->hidden_sc || !p->y))
+    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: null device address");
+  return PLK_OK;
+}
+
+static MokMxView view(uint64_t q, uint64_t sc, int64_t rows, int k, int ld_sc, bool per_expert) {
+  MokMxView v{};
+  v.q = (const uint8_t*)(uintptr_t)q;
+  v.sc = (const uint8_t*)(uintptr_t)sc;
+  v.rows = (int32_t)rows;
+  v.k = k;
+  v.ld_q = k;
+  v.ld_sc = ld_sc;
+  v.expert_pitch_q = per_expert ? rows * (int64_t)k : 0;
+  v.expert_pitch_sc = per_expert ? rows * (int64_t)ld_sc : 0;
+  return v;
+}
+
+extern "C" {
+
+int plk_mok_session_create(const void* image, size_t image_bytes, const plk_mok_link_info* link,
+                           plk_mok_session** out) {
+  if (!image || !link || !out) return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok_session_create: null argument");
+  if (link->struct_bytes != sizeof(plk_mok_link_info))
+    return plk_hip_set_error(PLK_E_VERSION, "plk_mok_session_create: link info struct size mismatch");
+  const uint32_t need[3][2] = {{link->framework_offset, (uint32_t)sizeof(MokFrameworkParams)},
+                               {link->gemm_offset, (uint32_t)sizeof(MokGemmResidue)},
+                               {link->act_offset, (uint32_t)sizeof(MokActResidue)}};
+  for (auto& n : need)
+    if (n[0] % 8 || n[0] + n[1] > link->params_bytes)
+      return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_session_create: params entry outside the image or misaligned");
+  if (link->threads != 256) return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_session_create: image must use 256 threads");
+  auto* s = new plk_mok_session;
+  s->link = *link;
+  int rc = plk_hip_module_load(image, image_bytes, &s->module);
+  if (rc == PLK_OK) rc = plk_hip_module_function(s->module, "pipelink_kernel", link->dyn_lds_bytes, &s->kernel);
+  for (int i = 0; i < 2 && rc == PLK_OK; ++i) {
+    rc = plk_hip_alloc(link->params_bytes, &s->params_dev[i]);
+    s->params_host[i].assign(link->params_bytes, 0xA5);  // differs from any real image: first call uploads
+  }
+  if (rc == PLK_OK) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    plk_hip_device_info info;
+    rc = plk_hip_device_info_get(dev, &info);
+    s->compute_units = info.compute_units;
+  }
+  if (rc != PLK_OK) {
+    plk_mok_session_destroy(s);
+    return rc;
+  }
+  *out = s;
+  return PLK_OK;
+}
+
+int plk_mok_session_destroy(plk_mok_session* s) {
+  if (!s) return PLK_OK;
+  int rc = PLK_OK;
+  for (uint64_t a : s->params_dev)
+    if (a) { int r = plk_hip_free(a); if (r) rc = r; }
+  if (s->module) { int r = plk_hip_module_unload(s->module); if (r) rc = r; }
+  delete s;
+  return rc;
+}
+
+int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass, void* stream) {
+  if (!s) return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok_forward: null session");
+  if (pass != 1 && pass != 2) return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok_forward: pass must be 1 or 2");
+  int rc = check_problem(p);
+  if (rc != PLK_OK) return rc;
+  if (p->routed_rows == 0) return PLK_OK;  // nothing routed to this rank
+
+  const int H = p->hidden, I = p->intermediate, E = p->num_experts;
+  MokFrameworkParams fw{};
+  fw.tokens_per_expert = (const int32_t*)(uintptr_t)p->tokens_per_expert;
+  fw.num_experts = E;
+  fw.op = pass == 1 ? MOK_GEMM_FWD_ROUTED_GATE_UP : MOK_GEMM_FWD_ROUTED_DOWN;
+  fw.num_col_tiles = pass == 1 ? (I + TILE_W / 2 - 1) / (TILE_W / 2) : (H + TILE_W - 1) / TILE_W;
+
+  MokGemmResidue g{};
+  g.x = view(p->x_q, p->x_sc, p->num_tokens, H, p->ld_sc_h, false);
+  g.hidden = view(p->hidden_q, p->hidden_sc, p->routed_rows, I, p->ld_sc_i, false);
+  g.w_gate = view(p->w_gate_q, p->w_gate_sc, I, H, p->ld_sc_h, true);
+  g.w_up = view(p->w_up_q, p->w_up_sc, I, H, p->ld_sc_h, true);
+  g.w_down = view(p->w_down_q, p->w_down_sc, H, I, p->ld_sc_i, true);
+  g.row_token = (const int32_t*)(uintptr_t)p->row_token;
+  g.y = (uint16_t*)(uintptr_t)p->y;
+  g.ld_y = H;
+
+  MokActResidue a{};
+  a.hidden_q = (uint8_t*)(uintptr_t)p->hidden_q;
+  a.hidden_sc = (uint8_t*)(uintptr_t)p->hidden_sc;
+  a.rows = p->routed_rows;
+  a.cols = I;
+  a.ld_q = I;
+  a.ld_sc = p->ld_sc_i;
+  a.swiglu_limit = p->swiglu_limit;
+
+  const int slot = pass - 1;
+  std::vector<unsigned char> image(s->link.params_bytes, 0);
+  std::memcpy(image.data() + s->link.framework_offset, &fw, sizeof fw);
+  std::memcpy(image.data() + s->link.gemm_offset, &g, sizeof g);
+  std::memcpy(image.data() + s->link.act_offset, &a, sizeof a);
+  if (image != s->params_host[slot]) {
+    rc = plk_hip_upload(s->params_dev[slot], image.data(), image.size(), stream);
+    if (rc != PLK_OK) return rc;
+    s->params_host[slot].swap(image);
+  }
+
+  // persistent grid: the solved occupancy on every CU, a multiple of the XCD count, but no
+  // more workgroups than there can be tiles
+  const int64_t max_row_tiles = (p->routed_rows + TILE_X - 1) / TILE_X + E;
+  const int64_t max_tiles = max_row_tiles * fw.num_col_tiles;
+  int64_t wgs = (int64_t)s->compute_units * s->link.workgroups_per_cu;
+  if (wgs > max_tiles) wgs = max_tiles;
+  wgs = (wgs + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
+  const uint32_t grid[3] = {(uint32_t)wgs, 1, 1};
+  const uint32_t block[3] = {s->link.threads, 1, 1};
+  return plk_hip_launch(s->kernel, grid, block, s->link.dyn_lds_bytes, stream, s->params_dev[slot]);
+}
+
+int plk_mok_forward(plk_mok_session* s, const plk_mok_problem* p, void* stream) {
+  int rc = plk_mok_forward_pass(s, p, 1, stream);
+  if (rc == PLK_OK) rc = plk_mok_forward_pass(s, p, 2, stream);
+  return rc;
+}
+
+}  // extern "C"
+
+// ---- MXFP8 block quantiser ---------------------------------------------------------------
+// One wave per row slice: each lane owns 4 consecutive elements, 8 lanes one 32-block.
+// OCP MX rule: scale byte = clamp(exponent_field(amax) - 8, 0, 254); elements are
+// e4m3_rne(clamp(v * 2^(127 - byte), +-448)).
+template <bool BF16>
+__global__ void __launch_bounds__(256) mxfp8_quantize_kernel(const void* __restrict__ src, int64_t rows, int k,
+                                                             uint8_t* __restrict__ dq, uint8_t* __restrict__ dsc,
+                                                             int ld_sc) {
+  const int blocks_per_row = k / 32;
+  const int64_t nblocks = rows * (int64_t)blocks_per_row;
+  const int sub = threadIdx.x & 7;
+  for (int64_t blk = (int64_t)blockIdx.x * 32 + (threadIdx.x >> 3); blk < nblocks; blk += (int64_t)gridDim.x * 32) {
+    const int64_t row = blk / blocks_per_row;
+    const int cb = (int)(blk - row * blocks_per_row);
+    const int64_t off = row * (int64_t)k + cb * 32 + sub * 4;
+    float v[4];
+    if (BF16) {
+      const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(src) + off);
+      v[0] = __uint_as_float(raw.x << 16);
+      v[1] = __uint_as_float(raw.x & 0xFFFF0000u);
+      v[2] = __uint_as_float(raw.y << 16);
+      v[3] = __uint_as_float(raw.y & 0xFFFF0000u);
+    } else {
+      const float4 raw = *reinterpret_cast<const float4*>(static_cast<const float*>(src) + off);
+      v[0] = raw.x; v[1] = raw.y; v[2] = raw.z; v[3] = raw.w;
+    }
+    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    amax = fmaxf(amax, __shfl_xor(amax, 1));
+    amax = fmaxf(amax, __shfl_xor(amax, 2));
+    amax = fmaxf(amax, __shfl_xor(amax, 4));
+    int e = (int)((__float_as_uint(amax) >> 23) & 0xFFu) - 8;
+    e = e < 0 ? 0 : e;
+    const float inv = __uint_as_float((uint32_t)(254 - e) << 23);
+    float s[4];
+    for (int j = 0; j < 4; ++j) s[j] = fminf(fmaxf(v[j] * inv, -448.0f), 448.0f);
+    int pk = 0;
+    pk = __builtin_amdgcn_cvt_pk_fp8_f32(s[0], s[1], pk, false);
+    pk = __builtin_amdgcn_cvt_pk_fp8_f32(s[2], s[3], pk, true);
+    *reinterpret_cast<uint32_t*>(dq + off) = (uint32_t)pk;
+    if (sub == 0) dsc[row * ld_sc + cb] = (uint8_t)e;
+    // zero the pad bytes of the scale row once per row
+    if (cb == 0 && sub == 1)
+      for (int c = blocks_per_row; c < ld_sc; ++c) dsc[row * ld_sc + c] = 0;
+  }
+}
+
+extern "C" int plk_mxfp8_quantize(uint64_t src, int src_is_bf16, int64_t rows, int32_t k, uint64_t dst_q,
+                                  uint64_t dst_sc, int32_t ld_sc, void* stream) {
+  if (rows < 0 || k <= 0 || k % 32 || ld_sc * 32 < k)
+    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mxfp8_quantize: k must be a positive multiple of 32 covered by ld_sc");
+  if (rows == 0) return PLK_OK;
+  if (!src || !dst_q || !dst_sc) return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mxfp8_quantize: null device address");
+  const int64_t nblocks = rows * (int64_t)(k / 32);
+  int64_t grid = (nblocks + 31) / 32;
+  if (grid > 65536) grid = 65536;
+  if (src_is_bf16)
+    mxfp8_quantize_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>(
+        (const void*)(uintptr_t)src, rows, k, (uint8_t*)(uintptr_t)dst_q, (uint8_t*)(uintptr_t)dst_sc, ld_sc);
+  else
+    mxfp8_quantize_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>(
+        (const void*)(uintptr_t)src, rows, k, (uint8_t*)(uintptr_t)dst_q, (uint8_t*)(uintptr_t)dst_sc, ld_sc);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return plk_hip_set_error(PLK_E_RESOURCE, hipGetErrorString(e));
+  return PLK_OK;
+}

@@ -1,0 +1,111 @@
+"""Host session of the routed-expert MXFP8 FFN forward (binding of ``include/plk_mok.h``).
+
+Plays the part of ``MoKHost`` in campaigns/mok/host/mok_port_host.py:72-289 for the forward
+pass: owns the loaded pipeline image, fills a problem record from torch tensors, launches
+on the current torch stream.  Tensors are only used as device memory.
+"""
+from __future__ import annotations
+
+import ctypes
+import json
+from ctypes import byref, c_void_p, sizeof
+
+import torch
+
+from .backend import MokLinkInfo, MokProblem, PlkError, check, load_library
+
+TILE_X = 128
+MX_BLOCK = 32
+
+
+def scale_pitch(k: int) -> int:
+    """Bytes per scale row: K/32 rounded up to a multiple of 4."""
+    return ((k // MX_BLOCK) + 3) // 4 * 4
+
+
+def link_info_from_json(link: dict) -> MokLinkInfo:
+    """Translate a ``link.json`` (pipec link output) into the C record the session wants."""
+    entries = {e["stage_id"]: e for e in link["params"]["entries"]}
+    return MokLinkInfo(struct_bytes=sizeof(MokLinkInfo), params_bytes=link["params"]["total_bytes"],
+                       framework_offset=entries["mok.framework"]["offset"], gemm_offset=entries["mok.gemm"]["offset"],
+                       act_offset=entries["mok.act"]["offset"], threads=link["threads"],
+                       dyn_lds_bytes=link["dyn_smem_bytes"], workgroups_per_cu=link.get("workgroups_per_cu", 1))
+
+
+class MoKSession:
+    def __init__(self, image: bytes, link: MokLinkInfo | dict | str):
+        if isinstance(link, str):
+            with open(link) as fh:
+                link = json.load(fh)
+        if isinstance(link, dict):
+            link = link_info_from_json(link)
+        self.lib = load_library()
+        self.link = link
+        handle = c_void_p()
+        buf = ctypes.create_string_buffer(image, len(image))
+        check(self.lib, self.lib.plk_mok_session_create(buf, len(image), byref(link), byref(handle)))
+        self._handle = handle
+
+    def close(self) -> None:
+        if self._handle:
+            check(self.lib, self.lib.plk_mok_session_destroy(self._handle))
+            self._handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    @staticmethod
+    def problem(*, x_q, x_sc, row_token, tokens_per_expert, w_gate_q, w_gate_sc, w_up_q, w_up_sc, w_down_q, w_down_sc,
+                hidden_q, hidden_sc, y, swiglu_limit: float = 7.0) -> MokProblem:
+        """Build the problem record from CUDA tensors (shapes checked here, contents by the library)."""
+        for name, t in dict(x_q=x_q, x_sc=x_sc, tokens_per_expert=tokens_per_expert, w_gate_q=w_gate_q,
+                            w_gate_sc=w_gate_sc, w_up_q=w_up_q, w_up_sc=w_up_sc, w_down_q=w_down_q,
+                            w_down_sc=w_down_sc, hidden_q=hidden_q, hidden_sc=hidden_sc, y=y).items():
+            if not t.is_cuda or not t.is_contiguous():
+                raise PlkError(3, f"{name} must be a contiguous device tensor")
+        t_rows, h = x_q.shape
+        e, i, h2 = w_gate_q.shape
+        r = y.shape[0]
+        if h2 != h or tuple(w_up_q.shape) != (e, i, h) or tuple(w_down_q.shape) != (e, h, i):
+            raise PlkError(3, "weight shapes disagree with x")
+        if tuple(hidden_q.shape) != (r, i) or y.shape[1] != h or y.dtype != torch.bfloat16:
+            raise PlkError(3, "hidden_q / y shapes disagree")
+        ldh, ldi = scale_pitch(h), scale_pitch(i)
+        if x_sc.shape[1] != ldh or w_gate_sc.shape[2] != ldh or w_up_sc.shape[2] != ldh or \
+                w_down_sc.shape[2] != ldi or hidden_sc.shape[1] != ldi:
+            raise PlkError(3, "scale pitch must be K/32 rounded up to a multiple of 4")
+        if tokens_per_expert.dtype != torch.int32 or (row_token is not None and row_token.dtype != torch.int32):
+            raise PlkError(3, "tokens_per_expert and row_token must be int32")
+        return MokProblem(struct_bytes=sizeof(MokProblem), num_tokens=t_rows, hidden=h, intermediate=i, num_experts=e,
+                          routed_rows=r, ld_sc_h=ldh, ld_sc_i=ldi, swiglu_limit=swiglu_limit,
+                          x_q=x_q.data_ptr(), x_sc=x_sc.data_ptr(),
+                          row_token=0 if row_token is None else row_token.data_ptr(),
+                          tokens_per_expert=tokens_per_expert.data_ptr(),
+                          w_gate_q=w_gate_q.data_ptr(), w_gate_sc=w_gate_sc.data_ptr(), w_up_q=w_up_q.data_ptr(),
+                          w_up_sc=w_up_sc.data_ptr(), w_down_q=w_down_q.data_ptr(), w_down_sc=w_down_sc.data_ptr(),
+                          hidden_q=hidden_q.data_ptr(), hidden_sc=hidden_sc.data_ptr(), y=y.data_ptr())
+
+    def forward(self, problem: MokProblem, stream: int | None = None, which: int = 0) -> None:
+        """Launch both passes (``which=0``) or one of them (1 = gate/up+SwiGLU+requant, 2 = down)."""
+        s = c_void_p(torch.cuda.current_stream().cuda_stream if stream is None else stream)
+        if which == 0:
+            check(self.lib, self.lib.plk_mok_forward(self._handle, byref(problem), s))
+        else:
+            check(self.lib, self.lib.plk_mok_forward_pass(self._handle, byref(problem), which, s))
+
+
+def mxfp8_quantize_device(src: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Quantise a 2-D fp32 or bf16 device tensor along its last axis on the GPU."""
+    if not src.is_cuda or not src.is_contiguous() or src.dim() != 2 or src.dtype not in (torch.float32, torch.bfloat16):
+        raise PlkError(3, "src must be a contiguous 2-D fp32/bf16 device tensor")
+    rows, k = src.shape
+    ld = scale_pitch(k)
+    q = torch.empty((rows, k), dtype=torch.uint8, device=src.device)
+    sc = torch.empty((rows, ld), dtype=torch.uint8, device=src.device)
+    lib = load_library()
+    check(lib, lib.plk_mxfp8_quantize(src.data_ptr(), int(src.dtype == torch.bfloat16), rows, k, q.data_ptr(),
+                                      sc.data_ptr(), ld, c_void_p(torch.cuda.current_stream().cuda_stream)))
+    return q, sc

@@ -1,0 +1,67 @@
+"""Seeded synthetic inputs of the routed-expert FFN forward.
+
+Draw order (CPU generator, seed given): router logits [T,E], x [T,H], then gate, up and
+down weights [E,N,K] scaled by 0.02, one expert at a time.  Routing is top-k of
+softmax(logits); the (token, slot) pairs are stably sorted by expert, which gives the
+routed-row order, ``tokens_per_expert`` and ``row_token``.  Follows the style of
+``MoKHost.new_inputs`` (campaigns/mok/host/mok_port_host.py:273-282), including its
+concentrated-routing generations that leave experts empty."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from .. import mxfp8
+
+
+@dataclass
+class MokInputs:
+    tokens_per_expert: torch.Tensor  # [E] int32
+    row_token: torch.Tensor          # [R] int32
+    x_q: torch.Tensor
+    x_sc: torch.Tensor
+    w_gate_q: torch.Tensor
+    w_gate_sc: torch.Tensor
+    w_up_q: torch.Tensor
+    w_up_sc: torch.Tensor
+    w_down_q: torch.Tensor
+    w_down_sc: torch.Tensor
+
+    def to(self, device):
+        return MokInputs(**{k: v.to(device) for k, v in self.__dict__.items()})
+
+
+def route(logits: torch.Tensor, top_k: int):
+    idx = torch.topk(torch.softmax(logits.float(), dim=-1), top_k, dim=-1).indices
+    flat = idx.reshape(-1)
+    order = torch.sort(flat, stable=True).indices
+    counts = torch.bincount(flat, minlength=logits.shape[1]).to(torch.int32)
+    return counts, (order // top_k).to(torch.int32)
+
+
+def generate(num_tokens: int, hidden: int, intermediate: int, num_experts: int, top_k: int, seed: int = 0,
+             concentrate: int = 0, quantize_device: torch.device | None = None) -> MokInputs:
+    """``concentrate`` > 0 routes every token to the first ``concentrate`` experts only (empty experts)."""
+    g = torch.Generator().manual_seed(seed)
+    logits = torch.randn(num_tokens, num_experts, generator=g)
+    if concentrate:
+        logits[:, concentrate:] = -1e9
+    x = torch.randn(num_tokens, hidden, generator=g)
+    counts, row_token = route(logits, top_k)
+    dev = quantize_device or torch.device("cpu")
+    x_q, x_sc = mxfp8.quantize(x.to(dev))
+
+    def weights(n, k):
+        qs, scs = [], []
+        for _ in range(num_experts):
+            w = torch.randn(n, k, generator=g) * 0.02
+            q, sc = mxfp8.quantize(w.to(dev))
+            qs.append(q)
+            scs.append(sc)
+        return torch.stack(qs), torch.stack(scs)
+
+    wg_q, wg_sc = weights(intermediate, hidden)
+    wu_q, wu_sc = weights(intermediate, hidden)
+    wd_q, wd_sc = weights(hidden, intermediate)
+    return MokInputs(counts.to(dev), row_token.to(dev), x_q, x_sc, wg_q, wg_sc, wu_q, wu_sc, wd_q, wd_sc)

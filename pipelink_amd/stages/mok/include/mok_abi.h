@@ -1,0 +1,109 @@
+/* MoK (routed-expert FFN) call ABI shared by the framework, GEMM and activation owners,
+ * host and device.  Plain C structs only; tile geometry of one owner reaches another only
+ * through the task records the framework fills in.
+ *
+ * Mirrors the role of campaigns/mok/port/include/mok_abi.h:15-17 (MokCounters),
+ * campaigns/mok/port/gemm/gemm_abi.h:7-13 (MokGemmTask) and
+ * campaigns/mok/port/act_gptoss/act_abi.h:8-15 (MokActTask).  Field sets differ: TMA
+ * descriptors and CLC/cluster ranks have no gfx950 counterpart, and one task here is one
+ * workgroup tile whose gate and up halves are produced together so that the activation
+ * runs on the accumulator instead of on a bf16 round trip through HBM. */
+#ifndef PIPELINK_MOK_ABI_H
+#define PIPELINK_MOK_ABI_H
+
+#include <stdint.h>
+
+#ifndef MOKCOUNTERS_DEFINED
+#define MOKCOUNTERS_DEFINED
+typedef struct MokCounters {
+  int32_t* base; /* counter workspace lent by the framework to every op call */
+} MokCounters;
+#endif
+
+/* op codes keep the reference's names; GATE and UP of one tile are issued as one task */
+enum {
+  MOK_GEMM_FWD_ROUTED_GATE_UP = 3, /* = MOK_GEMM_FWD_ROUTED_GATE of the reference */
+  MOK_GEMM_FWD_ROUTED_DOWN = 5
+};
+enum { MOK_ACT_FWD_ROUTED = 1 };
+
+#ifndef MOKGEMMTASK_DEFINED
+#define MOKGEMMTASK_DEFINED
+typedef struct MokGemmTask {
+  int32_t op;        /* MOK_GEMM_FWD_ROUTED_GATE_UP or MOK_GEMM_FWD_ROUTED_DOWN */
+  int32_t expert;    /* local expert whose weights this tile multiplies */
+  int32_t row_begin; /* first routed row of the tile */
+  int32_t row_end;   /* one past the expert's last routed row; rows >= row_end are padding */
+  int32_t col_begin; /* first output column of the tile (per weight matrix) */
+  int32_t task_idx;  /* running index of the tile in the schedule */
+  uint32_t flags;
+} MokGemmTask;
+#endif
+
+#ifndef MOKACTTASK_DEFINED
+#define MOKACTTASK_DEFINED
+typedef struct MokActTask {
+  int32_t op;        /* MOK_ACT_FWD_ROUTED */
+  int32_t row_begin, row_end, col_begin;
+  int32_t task_idx;
+  uint32_t flags;
+} MokActTask;
+#endif
+
+/* One MXFP8 operand: e4m3 codes [rows, k] (row pitch ld_q bytes) and e8m0 scales
+ * [rows, ld_sc] (one byte per 32 k-elements, ld_sc a multiple of 4).  Weights carry an
+ * expert pitch on both. */
+typedef struct MokMxView {
+  const uint8_t* q;
+  const uint8_t* sc;
+  int64_t expert_pitch_q;
+  int64_t expert_pitch_sc;
+  int32_t rows; /* rows per expert for weights, total rows for activations */
+  int32_t k;
+  int32_t ld_q;
+  int32_t ld_sc;
+} MokMxView;
+
+/* Residue of the GEMM owner: every device address and extent its exports read. */
+typedef struct MokGemmResidue {
+  MokMxView x;       /* activations in token order [T, H] */
+  MokMxView hidden;  /* SwiGLU output in routed-row order [R, I] (read by the down GEMM) */
+  MokMxView w_gate;  /* [E, I, H] */
+  MokMxView w_up;    /* [E, I, H] */
+  MokMxView w_down;  /* [E, H, I] */
+  const int32_t* row_token; /* [R] routed row -> token row of x; null = identity */
+  uint16_t* y;       /* bf16 [R, H] */
+  int32_t ld_y;      /* elements */
+  int32_t reserved;
+} MokGemmResidue;
+
+/* Residue of the activation owner. */
+typedef struct MokActResidue {
+  uint8_t* hidden_q;  /* e4m3 [R, I] */
+  uint8_t* hidden_sc; /* e8m0 [R, ld_sc] */
+  int32_t rows, cols, ld_q, ld_sc;
+  float swiglu_limit;
+  int32_t reserved;
+} MokActResidue;
+
+/* Params of the framework role: the schedule. */
+typedef struct MokFrameworkParams {
+  const int32_t* tokens_per_expert; /* [E] */
+  int32_t* expert_row_begin;        /* [E+1] exclusive prefix sum of tokens_per_expert (workspace) */
+  int32_t* expert_tile_begin;       /* [E+1] exclusive prefix sum of row tiles (workspace) */
+  int32_t num_experts;
+  int32_t op;                       /* which GEMM this launch runs */
+  int32_t num_col_tiles;
+  int32_t reserved;
+} MokFrameworkParams;
+
+/* First argument of every owner export (pack/include/pipelink/host_view.h in the reference). */
+#ifndef PIPELINK_HOST_VIEW_DEFINED
+#define PIPELINK_HOST_VIEW_DEFINED
+typedef struct pipelink_host_view {
+  const void* residue;
+  const void* scalars;
+} pipelink_host_view;
+#endif
+
+#endif

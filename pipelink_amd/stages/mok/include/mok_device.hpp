@@ -1,0 +1,65 @@
+// Device-side helpers shared by the MoK stage sources: vector types, the MFMA wrapper and
+// the contract that says where one element of the grouped-GEMM accumulator lives.
+#ifndef PIPELINK_MOK_DEVICE_HPP
+#define PIPELINK_MOK_DEVICE_HPP
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "mok_abi.h"
+
+namespace mok {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// ---- tile geometry published by the GEMM owner (facts mok.gemm.*) -------------------
+// One workgroup tile = TILE_X routed rows x TILE_W weight rows, 4 waves as 2 (weights) x 2
+// (rows).  For the gate/up op the weight rows are TILE_W/2 gate columns followed by the
+// same TILE_W/2 up columns, so gate and up of one output element meet in one register.
+constexpr int TILE_X = 128;
+constexpr int TILE_W = 256;
+constexpr int K_STEP = 64;      // contraction elements per ring stage = one MFMA 32x32x64
+constexpr int WFRAGS = 4;       // 32-row weight fragments per wave
+constexpr int XFRAGS = 2;       // 32-row activation fragments per wave
+constexpr int THREADS = 256;
+constexpr int STAGE_X_BYTES = TILE_X * K_STEP;
+constexpr int STAGE_W_BYTES = TILE_W * K_STEP;
+constexpr int STAGE_BYTES = STAGE_X_BYTES + STAGE_W_BYTES;  // 24576
+
+// fp32 accumulator of one wave: [weight fragment][row fragment] MFMA 32x32 C tiles.
+// Element (reg r, lane l) of tile (a, b) is
+//   weight row  = wrow0(a) + 8*(r/4) + 4*(l/32) + r%4      (output column)
+//   routed row  = xrow0(b) + l%32
+// with wrow0/xrow0 below.  This is the placement the activation owner imports.
+struct AccFrag {
+  v16f v[WFRAGS][XFRAGS];
+};
+
+__device__ __forceinline__ int wave_w(int wave) { return wave & 1; }
+__device__ __forceinline__ int wave_x(int wave) { return wave >> 1; }
+// first tile-local weight row of fragment a for this wave (rows [0,128) | [128,256))
+__device__ __forceinline__ int wrow0(int wave, int a) {
+  return (a < 2 ? 0 : TILE_W / 2) + wave_w(wave) * 64 + (a & 1) * 32;
+}
+__device__ __forceinline__ int xrow0(int wave, int b) { return wave_x(wave) * 64 + b * 32; }
+
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+// 16 bytes per lane, global -> LDS, lane i lands at lds + 16*i
+__device__ __forceinline__ void load16_to_lds(const uint8_t* g, unsigned char* lds) {
+  __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)lds, 16, 0, 0);
+}
+
+__device__ __forceinline__ float bf16_round(float x) {
+  uint32_t u = __float_as_uint(x);
+  u = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
+  return __uint_as_float(u);
+}
+
+}  // namespace mok
+
+#endif
