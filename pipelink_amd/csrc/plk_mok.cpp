@@ -14,7 +14,7 @@
 extern "C" int plk_hip_set_error(int code, const char* what);
 
 namespace {
-constexpr int TILE_X = 128;  // routed rows per workgroup tile   (fact mok.gemm.TILE_X)
+constexpr int TILE_X = 256;  // routed rows per workgroup tile   (fact mok.gemm.TILE_X)
 constexpr int TILE_W = 256;  // weight rows per workgroup tile   (fact mok.gemm.TILE_W)
 constexpr int K_STEP = 64;
 constexpr int MAX_EXPERTS = 256;
@@ -74,7 +74,7 @@ int plk_mok_session_create(const void* image, size_t image_bytes, const plk_mok_
   for (auto& n : need)
     if (n[0] % 8 || n[0] + n[1] > link->params_bytes)
       return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_session_create: params entry outside the image or misaligned");
-  if (link->threads != 256) return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_session_create: image must use 256 threads");
+  if (link->threads != 512) return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_session_create: image must use 512 threads");
   auto* s = new plk_mok_session;
   s->link = *link;
   int rc = plk_hip_module_load(image, image_bytes, &s->module);

@@ -9,14 +9,17 @@
 // four consecutive output columns of one routed row, which is what the requantising
 // epilogue and the bf16 store want.
 //
-// Ring: `depth` LDS stages of 24 KB, each holding 64 contraction bytes of 128 routed rows
-// and 256 weight rows in [16-byte chunk][row] order: a wave's global_load_lds of one chunk
-// of 64 consecutive rows lands contiguously, and a fragment read (32 lanes, 16 bytes each,
-// consecutive rows) is contiguous too, so neither side has bank conflicts.  The depth is a
-// link-time handle; the ring offset inside the workgroup's dynamic LDS is another.
+// Ring: `depth` LDS slots of 66 KB.  A slot holds 128 contraction bytes of 256 routed rows
+// and of 256 weight rows, row-major (one 128-byte cache line per row), followed by one
+// dword of block scales (4 x e8m0) per row.  One global_load_lds_dwordx4 moves 8 rows:
+// eight lanes cover the 128 contiguous bytes of a row, so every L2 request is a full line.
+// The eight 16-byte chunks of a row are stored at position chunk ^ ((row / 2) % 8), which
+// makes a fragment read (32 consecutive rows, one chunk each) touch 16 different 16-byte
+// bank groups per 16 lanes.  The depth is a link-time handle; the ring offset inside the
+// workgroup's dynamic LDS is another.
 #include "../include/mok_device.hpp"
 
-extern "C" __device__ int pipelink_mok_gemm_depth();  // ring stages (2..6), bound at link time
+extern "C" __device__ int pipelink_mok_gemm_depth();  // ring slots (2 or 3), bound at link time
 extern "C" __device__ int pipelink_mok_gemm_arena();  // byte offset of the ring in dynamic LDS
 
 extern __shared__ __attribute__((aligned(1024))) unsigned char pipelink_smem[];
@@ -24,32 +27,44 @@ extern __shared__ __attribute__((aligned(1024))) unsigned char pipelink_smem[];
 namespace mok_gemm_owner {
 using namespace mok;
 
-constexpr int LOADS_PER_STEP = STAGE_BYTES / (THREADS * 16);  // 6 direct-to-LDS loads per lane
+constexpr int WAVES = THREADS / 64;
+constexpr int X_GROUPS = TILE_X / 8 / WAVES;  // 8-row load groups per wave (4)
+constexpr int W_GROUPS = TILE_W / 8 / WAVES;  // (4)
+constexpr int LOADS_PER_SLOT = X_GROUPS + W_GROUPS + 1;  // + one dword of scales per lane
 
 struct Loader {
-  const uint8_t* xsrc;  // this lane's routed row, at this wave's first chunk
-  const uint8_t* wsrc;  // this lane's weight row
-  int xdst;             // stage-relative LDS byte offsets of the wave's first chunk
-  int wdst;
+  const uint8_t* xsrc[X_GROUPS];  // this lane's 16 bytes of its row in each group, at k = 0
+  const uint8_t* wsrc[W_GROUPS];
+  const uint8_t* scsrc;           // scale row of this thread's row (threads 0..255 rows, 256..511 weights)
+  int chunk_byte;                 // byte offset inside the 128-byte line this lane fetches in even groups
+  int xdst, wdst, scdst;          // slot-relative LDS byte offsets of the wave's first group
 };
 
-__device__ __forceinline__ void issue_stage(const Loader& ld, unsigned char* stage, int kbyte) {
-  // activations: 2 chunks per wave; weights: 4 chunks per wave
-  load16_to_lds(ld.xsrc + kbyte, stage + ld.xdst);
-  load16_to_lds(ld.xsrc + kbyte + 16, stage + ld.xdst + TILE_X * 16);
+__device__ __forceinline__ int swizzle(int row) { return (row >> 1) & 7; }
+
+// Issue one slot.  k_left = contraction bytes from this slot's start to the end of the row:
+// the last slot of a K that is not a multiple of 128 only fetches the chunks that exist.
+__device__ __forceinline__ void issue_slot(const Loader& ld, unsigned char* slot, int kbyte, int k_left) {
+  // group j starts at tile row 8 * (4 * wave + j): odd groups flip bit 2 of the swizzle, so
+  // the lane's chunk there is the even-group chunk with bit 2 (64 bytes) flipped
 #pragma unroll
-  for (int c = 0; c < 4; ++c)
-    load16_to_lds(ld.wsrc + kbyte + 16 * c, stage + ld.wdst + c * TILE_W * 16);
+  for (int j = 0; j < X_GROUPS; ++j)
+    if ((ld.chunk_byte ^ ((j & 1) << 6)) < k_left) load16_to_lds(ld.xsrc[j] + kbyte, slot + ld.xdst + j * 1024);
+#pragma unroll
+  for (int j = 0; j < W_GROUPS; ++j)
+    if ((ld.chunk_byte ^ ((j & 1) << 6)) < k_left) load16_to_lds(ld.wsrc[j] + kbyte, slot + ld.wdst + j * 1024);
+  load4_to_lds(ld.scsrc + (kbyte >> 5), slot + ld.scdst);
 }
 
 // MFMA 32x32x64 f8f6f4 operand of lane (row = lane % 32, half = lane / 32): registers 0-3
 // hold 16 bytes of the step's first 32-element block, registers 4-7 16 bytes of its second
 // block; the scale of block 0 is taken from lanes 0-31 and that of block 1 from lanes 32-63
-// (measured on gfx950 with a one-instruction probe).  So a lane reads chunk `half` and
-// chunk `half + 2` of its row.
-__device__ __forceinline__ v8i read_frag(const unsigned char* chunk_lo, int plane_bytes) {
-  const v4i lo = *reinterpret_cast<const v4i*>(chunk_lo);
-  const v4i hi = *reinterpret_cast<const v4i*>(chunk_lo + 2 * plane_bytes);
+// (measured on gfx950 with a one-instruction probe).  So in 64-byte step s of a slot a lane
+// reads chunks 4s + half and 4s + half + 2 of its row; with the XOR swizzle these are the
+// step-0 offsets with bit 6 (step) and bit 5 (second block) flipped.
+__device__ __forceinline__ v8i read_frag(const unsigned char* slot, int off) {
+  const v4i lo = *reinterpret_cast<const v4i*>(slot + off);
+  const v4i hi = *reinterpret_cast<const v4i*>(slot + (off ^ 32));
   v8i r;
   r.s0 = lo.x; r.s1 = lo.y; r.s2 = lo.z; r.s3 = lo.w;
   r.s4 = hi.x; r.s5 = hi.y; r.s6 = hi.z; r.s7 = hi.w;
@@ -71,37 +86,15 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
 }
 
-template <int DEPTH>
-struct Ring {
-  unsigned char* base;
-  int slot;  // stage the next step consumes
-  int fill;  // stage the next issued load fills
-};
-
-// One 64-element contraction step: wait for its stage, refill the stage freed by the
-// previous step, read 6 fragments, issue 8 MFMAs.
-template <int DEPTH, bool ODD>
-__device__ __forceinline__ void step(const Loader& ld, Ring<DEPTH>& rs, int i, int nk, const int (&xoff)[XFRAGS],
-                                     const int (&woff)[WFRAGS], const int (&sx)[XFRAGS], const int (&sw)[WFRAGS],
-                                     AccFrag& acc) {
-  // Loads younger than stage i's: the stages i+1 .. i+DEPTH-2 and the pair's batch of scale
-  // dwords, which is issued at the top of the even step -- after stage i's loads except for
-  // the odd step of a two-stage ring, whose stage is only issued inside the even step.
-  constexpr int YOUNGER_SCALES = (ODD && DEPTH == 2) ? 0 : XFRAGS + WFRAGS;
-  if (i + DEPTH - 2 < nk)
-    wait_vmcnt<(DEPTH - 2) * LOADS_PER_STEP + YOUNGER_SCALES>();
-  else
-    wait_vmcnt<0>();
-  wg_barrier();
-  if (i + DEPTH - 1 < nk) issue_stage(ld, rs.base + rs.fill * STAGE_BYTES, (i + DEPTH - 1) * K_STEP);
-  rs.fill = rs.fill + 1 == DEPTH ? 0 : rs.fill + 1;
-  const unsigned char* stage = rs.base + rs.slot * STAGE_BYTES;
-  rs.slot = rs.slot + 1 == DEPTH ? 0 : rs.slot + 1;
+template <bool ODD>
+__device__ __forceinline__ void mma_step(const unsigned char* slot, const int (&xoff)[XFRAGS],
+                                         const int (&woff)[WFRAGS], const int (&sx)[XFRAGS],
+                                         const int (&sw)[WFRAGS], AccFrag& acc) {
   v8i xf[XFRAGS], wf[WFRAGS];
 #pragma unroll
-  for (int b = 0; b < XFRAGS; ++b) xf[b] = read_frag(stage + xoff[b], TILE_X * 16);
+  for (int b = 0; b < XFRAGS; ++b) xf[b] = read_frag(slot, xoff[b] ^ (ODD ? 64 : 0));
 #pragma unroll
-  for (int a = 0; a < WFRAGS; ++a) wf[a] = read_frag(stage + woff[a], TILE_W * 16);
+  for (int a = 0; a < WFRAGS; ++a) wf[a] = read_frag(slot, woff[a] ^ (ODD ? 64 : 0));
 #pragma unroll
   for (int a = 0; a < WFRAGS; ++a)
 #pragma unroll
@@ -119,45 +112,66 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   const int half = lane >> 5;
   const bool gate_up = t.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
   const MokMxView& act = gate_up ? g.x : g.hidden;
-  const int nk = act.k / K_STEP;
+  const int K = act.k;
+  const int nslots = (K + K_SLOT - 1) / K_SLOT;
   unsigned char* ring = pipelink_smem + pipelink_mok_gemm_arena();
 
   // ---- loader addresses (fixed for the tile) ---------------------------------------
+  // lane -> (row lane/8 of an 8-row group, LDS position lane%8); it fetches the chunk that
+  // belongs at that position
   Loader ld;
   {
-    int row = t.row_begin + (wave & 1) * 64 + lane;
-    row = row < t.row_end ? row : t.row_end - 1;
-    const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
-    ld.xsrc = act.q + (int64_t)src * act.ld_q + (wave >> 1) * 32;
-    ld.xdst = (wave >> 1) * 2 * (TILE_X * 16) + (wave & 1) * 1024;
-    const int wl = wave * 64 + lane;  // tile-local weight row
-    const MokMxView& wv = gate_up ? (wave < 2 ? g.w_gate : g.w_up) : g.w_down;
-    int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
-    col = col < wv.rows ? col : wv.rows - 1;
-    ld.wsrc = wv.q + (int64_t)t.expert * wv.expert_pitch_q + (int64_t)col * wv.ld_q;
-    ld.wdst = STAGE_X_BYTES + wave * 1024;
+    const int lrow = lane >> 3;
+    const int pos = lane & 7;
+    ld.chunk_byte = 16 * (pos ^ swizzle(lrow));
+    static_assert(X_GROUPS % 2 == 0 && W_GROUPS % 2 == 0, "a wave's first group must start at a multiple of 16 rows");
+#pragma unroll
+    for (int j = 0; j < X_GROUPS; ++j) {
+      const int trow = (wave * X_GROUPS + j) * 8 + lrow;  // tile-local routed row
+      int row = t.row_begin + trow;
+      row = row < t.row_end ? row : t.row_end - 1;
+      const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
+      ld.xsrc[j] = act.q + (int64_t)src * act.ld_q + 16 * (pos ^ swizzle(trow));
+    }
+    ld.xdst = wave * X_GROUPS * 1024;
+    const MokMxView& wv = gate_up ? (wave < WAVES / 2 ? g.w_gate : g.w_up) : g.w_down;
+#pragma unroll
+    for (int j = 0; j < W_GROUPS; ++j) {
+      const int wl = (wave * W_GROUPS + j) * 8 + lrow;  // tile-local weight row
+      int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
+      col = col < wv.rows ? col : wv.rows - 1;
+      ld.wsrc[j] = wv.q + (int64_t)t.expert * wv.expert_pitch_q + (int64_t)col * wv.ld_q + 16 * (pos ^ swizzle(wl));
+    }
+    ld.wdst = SLOT_X_BYTES + wave * W_GROUPS * 1024;
+    // scales: thread tid < 256 fetches routed row tid's dword, the others weight row tid - 256
+    if (tid < TILE_X) {
+      int row = t.row_begin + tid;
+      row = row < t.row_end ? row : t.row_end - 1;
+      const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
+      ld.scsrc = act.sc + (int64_t)src * act.ld_sc;
+    } else {
+      const int wl = tid - TILE_X;
+      const MokMxView& sv = gate_up ? (wl < TILE_W / 2 ? g.w_gate : g.w_up) : g.w_down;
+      int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
+      col = col < sv.rows ? col : sv.rows - 1;
+      ld.scsrc = sv.sc + (int64_t)t.expert * sv.expert_pitch_sc + (int64_t)col * sv.ld_sc;
+    }
+    ld.scdst = SLOT_X_BYTES + SLOT_W_BYTES + wave * 256;
   }
 
-  // ---- per-fragment scale rows and LDS read offsets --------------------------------
-  const uint8_t* xsc[XFRAGS];
-  const uint8_t* wsc[WFRAGS];
-  int xoff[XFRAGS], woff[WFRAGS];
+  // ---- per-fragment LDS read offsets (step 0, first block) ---------------------------
+  int xoff[XFRAGS], woff[WFRAGS], xscoff[XFRAGS], wscoff[WFRAGS];
 #pragma unroll
   for (int b = 0; b < XFRAGS; ++b) {
-    int row = t.row_begin + xrow0(wave, b) + r32;
-    row = row < t.row_end ? row : t.row_end - 1;
-    const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
-    xsc[b] = act.sc + (int64_t)src * act.ld_sc;
-    xoff[b] = half * (TILE_X * 16) + (xrow0(wave, b) + r32) * 16;
+    const int row = xrow0(wave, b) + r32;
+    xoff[b] = row * K_SLOT + 16 * (half ^ swizzle(row));
+    xscoff[b] = SLOT_X_BYTES + SLOT_W_BYTES + row * 4;
   }
 #pragma unroll
   for (int a = 0; a < WFRAGS; ++a) {
     const int wl = wrow0(wave, a) + r32;
-    const MokMxView& wv = gate_up ? (a < 2 ? g.w_gate : g.w_up) : g.w_down;
-    int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
-    col = col < wv.rows ? col : wv.rows - 1;
-    wsc[a] = wv.sc + (int64_t)t.expert * wv.expert_pitch_sc + (int64_t)col * wv.ld_sc;
-    woff[a] = STAGE_X_BYTES + half * (TILE_W * 16) + wl * 16;
+    woff[a] = SLOT_X_BYTES + wl * K_SLOT + 16 * (half ^ swizzle(wl));
+    wscoff[a] = SLOT_X_BYTES + SLOT_W_BYTES + TILE_X * 4 + wl * 4;
   }
 
 #pragma unroll
@@ -167,34 +181,35 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc.v[a][b][r] = 0.0f;
 
-  // ---- prologue: scales of the first pair, then depth-1 stages -----------------------
-  int sx[XFRAGS], sw[WFRAGS], sx_next[XFRAGS], sw_next[WFRAGS];
-  const int npairs = (nk + 1) >> 1;
-#pragma unroll
-  for (int b = 0; b < XFRAGS; ++b) sx[b] = (int)(*reinterpret_cast<const uint32_t*>(xsc[b]) >> (8 * half));
-#pragma unroll
-  for (int a = 0; a < WFRAGS; ++a) sw[a] = (int)(*reinterpret_cast<const uint32_t*>(wsc[a]) >> (8 * half));
+  // ---- prologue: fill depth-1 slots ---------------------------------------------------
 #pragma unroll
   for (int s = 0; s < DEPTH - 1; ++s)
-    if (s < nk) issue_stage(ld, ring + s * STAGE_BYTES, s * K_STEP);
+    if (s < nslots) issue_slot(ld, ring + s * SLOT_BYTES, s * K_SLOT, K - s * K_SLOT);
 
-  Ring<DEPTH> rs{ring, 0, DEPTH - 1};
-  for (int p = 0; p < npairs; ++p) {
-    // Scale bytes of the next 128-element pair: one dword per row.  Issued before this
-    // pair's stage loads so that waiting for them never drains younger stage loads; the
-    // last pair re-reads its own dword to keep the number of loads in flight uniform.
-    const int pn = p + 1 < npairs ? p + 1 : p;
+  int cur = 0;           // slot the next iteration consumes
+  int fill = DEPTH - 1;  // slot the next issued load fills
+  for (int i = 0; i < nslots; ++i) {
+    // loads younger than slot i's: the slots i+1 .. i+DEPTH-2
+    if (i + DEPTH - 2 < nslots)
+      wait_vmcnt<(DEPTH - 2) * LOADS_PER_SLOT>();
+    else
+      wait_vmcnt<0>();
+    wg_barrier();  // slot i has landed for every wave; everyone is done reading slot i-1
+    if (i + DEPTH - 1 < nslots)
+      issue_slot(ld, ring + fill * SLOT_BYTES, (i + DEPTH - 1) * K_SLOT, K - (i + DEPTH - 1) * K_SLOT);
+    fill = fill + 1 == DEPTH ? 0 : fill + 1;
+    const unsigned char* slot = ring + cur * SLOT_BYTES;
+    cur = cur + 1 == DEPTH ? 0 : cur + 1;
+
+    // block scales of the slot: lanes of the upper half use blocks 1 and 3, shifted down
+    // into bytes 0 and 2 where the MFMA's op_sel picks them
+    int sx[XFRAGS], sw[WFRAGS];
 #pragma unroll
-    for (int b = 0; b < XFRAGS; ++b) sx_next[b] = (int)*reinterpret_cast<const uint32_t*>(xsc[b] + 4 * pn);
+    for (int b = 0; b < XFRAGS; ++b) sx[b] = (int)(*reinterpret_cast<const uint32_t*>(slot + xscoff[b]) >> (8 * half));
 #pragma unroll
-    for (int a = 0; a < WFRAGS; ++a) sw_next[a] = (int)*reinterpret_cast<const uint32_t*>(wsc[a] + 4 * pn);
-    step<DEPTH, false>(ld, rs, 2 * p, nk, xoff, woff, sx, sw, acc);
-    if (2 * p + 1 < nk) step<DEPTH, true>(ld, rs, 2 * p + 1, nk, xoff, woff, sx, sw, acc);
-    // lanes of the upper half use blocks 1 and 3: shift them down into bytes 0 and 2
-#pragma unroll
-    for (int b = 0; b < XFRAGS; ++b) sx[b] = (int)((uint32_t)sx_next[b] >> (8 * half));
-#pragma unroll
-    for (int a = 0; a < WFRAGS; ++a) sw[a] = (int)((uint32_t)sw_next[a] >> (8 * half));
+    for (int a = 0; a < WFRAGS; ++a) sw[a] = (int)(*reinterpret_cast<const uint32_t*>(slot + wscoff[a]) >> (8 * half));
+    mma_step<false>(slot, xoff, woff, sx, sw, acc);
+    if (K - i * K_SLOT > 64) mma_step<true>(slot, xoff, woff, sx, sw, acc);
   }
   wg_barrier();  // ring free for the next tile
 }
@@ -237,12 +252,9 @@ extern "C" __device__ void mok_gemm_fwd(const void* view, const MokGemmTask* tas
   (void)counters;
   (void)phase;
   const auto& g = *static_cast<const MokGemmResidue*>(static_cast<const pipelink_host_view*>(view)->residue);
-  switch (pipelink_mok_gemm_depth()) {
-    case 2: mok_gemm_owner::mainloop<2>(g, *task, *acc); break;
-    case 3: mok_gemm_owner::mainloop<3>(g, *task, *acc); break;
-    case 4: mok_gemm_owner::mainloop<4>(g, *task, *acc); break;
-    case 5: mok_gemm_owner::mainloop<5>(g, *task, *acc); break;
-    default: mok_gemm_owner::mainloop<6>(g, *task, *acc); break;
-  }
+  if (pipelink_mok_gemm_depth() == 2)
+    mok_gemm_owner::mainloop<2>(g, *task, *acc);
+  else
+    mok_gemm_owner::mainloop<3>(g, *task, *acc);  // needs 3 x 66 KB: beyond one CU's LDS at this tile size
   if (task->op == MOK_GEMM_FWD_ROUTED_DOWN) mok_gemm_owner::store_down(g, *task, *acc);
 }

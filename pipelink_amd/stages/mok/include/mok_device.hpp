@@ -15,18 +15,20 @@ typedef int v2i __attribute__((ext_vector_type(2)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 // ---- tile geometry published by the GEMM owner (facts mok.gemm.*) -------------------
-// One workgroup tile = TILE_X routed rows x TILE_W weight rows, 4 waves as 2 (weights) x 2
-// (rows).  For the gate/up op the weight rows are TILE_W/2 gate columns followed by the
-// same TILE_W/2 up columns, so gate and up of one output element meet in one register.
-constexpr int TILE_X = 128;
+// One workgroup tile = TILE_X routed rows x TILE_W weight rows, 8 waves as 4 (rows) x 2
+// (weights), each wave a 64 x 128 sub-tile.  For the gate/up op the weight rows are
+// TILE_W/2 gate columns followed by the same TILE_W/2 up columns, so gate and up of one
+// output element meet in one register.
+constexpr int TILE_X = 256;
 constexpr int TILE_W = 256;
-constexpr int K_STEP = 64;      // contraction elements per ring stage = one MFMA 32x32x64
+constexpr int K_SLOT = 128;     // contraction bytes per ring slot = two MFMA 32x32x64 steps
 constexpr int WFRAGS = 4;       // 32-row weight fragments per wave
 constexpr int XFRAGS = 2;       // 32-row activation fragments per wave
-constexpr int THREADS = 256;
-constexpr int STAGE_X_BYTES = TILE_X * K_STEP;
-constexpr int STAGE_W_BYTES = TILE_W * K_STEP;
-constexpr int STAGE_BYTES = STAGE_X_BYTES + STAGE_W_BYTES;  // 24576
+constexpr int THREADS = 512;
+constexpr int SLOT_X_BYTES = TILE_X * K_SLOT;
+constexpr int SLOT_W_BYTES = TILE_W * K_SLOT;
+constexpr int SLOT_SCALE_BYTES = (TILE_X + TILE_W) * 4;  // one dword (4 block scales) per row
+constexpr int SLOT_BYTES = SLOT_X_BYTES + SLOT_W_BYTES + SLOT_SCALE_BYTES;  // 67584
 
 // fp32 accumulator of one wave: [weight fragment][row fragment] MFMA 32x32 C tiles.
 // Element (reg r, lane l) of tile (a, b) is
@@ -45,13 +47,16 @@ __device__ __forceinline__ int wrow0(int wave, int a) {
 }
 __device__ __forceinline__ int xrow0(int wave, int b) { return wave_x(wave) * 64 + b * 32; }
 
-
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
 // 16 bytes per lane, global -> LDS, lane i lands at lds + 16*i
 __device__ __forceinline__ void load16_to_lds(const uint8_t* g, unsigned char* lds) {
   __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)lds, 16, 0, 0);
+}
+// 4 bytes per lane, lane i lands at lds + 4*i
+__device__ __forceinline__ void load4_to_lds(const uint8_t* g, unsigned char* lds) {
+  __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)lds, 4, 0, 0);
 }
 
 __device__ __forceinline__ float bf16_round(float x) {
