@@ -1,0 +1,195 @@
+#!/usr/bin/env python3
+"""Benchmark of the routed-expert MXFP8 FFN forward (gate/up grouped GEMM -> clamped SwiGLU ->
+MXFP8 requant -> down grouped GEMM -> bf16) on one MI355X.
+
+One step = one forward over the whole batch: T=8192 tokens, d_model=d_ff=2880, 32 experts,
+top-4 routing (32768 routed rows), inputs already resident in HBM.  Prints ONE JSON line:
+metric = MXFP8 grouped-GEMM TFLOP/s on the algorithmic (unpadded) flop count
+2*R*H*I*3 = 1.6307e12 per forward, plus
+  roofline      -- the gate/up pass (the dominant kernel) timed with HIP events on its launch
+                   stream, against the 5.0 PFLOP/s dense FP8 MFMA peak;
+  cpu_baseline  -- the CPU oracle (torch fp32 dequant-then-matmul) timed on the host cores on
+                   the first 1024 tokens of the same inputs;
+  linked_over_one_unit -- paired ABBA/BAAB timing of the linked image against the one-unit
+                   control (evaluator/harness/parity/example.py:104-166 in the reference)."""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+T, H, I, E, TOPK = 8192, 2880, 2880, 32, 4
+FLOPS_GATE_UP = 2.0 * T * TOPK * H * I * 2
+FLOPS_DOWN = 2.0 * T * TOPK * I * H
+FLOPS_TOTAL = FLOPS_GATE_UP + FLOPS_DOWN
+PEAK_FP8_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
+
+
+def make_inputs(dev, seed=0):
+    """Seeded config-3 inputs: CPU generator, draw order logits, x, Wg, Wu, Wd (one expert at a
+    time); quantised on the device (bit-exact with the host rule) into 128-byte-pitched rows."""
+    import torch
+    from pipelink_amd.host import mok_inputs
+    from pipelink_amd.host.mok import code_pitch, mxfp8_quantize_device
+
+    g = torch.Generator().manual_seed(seed)
+    logits = torch.randn(T, E, generator=g)
+    x = torch.randn(T, H, generator=g)
+    counts, row_token = mok_inputs.route(logits, TOPK)
+    x_q, x_sc = mxfp8_quantize_device(x.to(dev), code_pitch(H))
+
+    def weights(n, k):
+        qs, scs = [], []
+        for _ in range(E):
+            w = torch.randn(n, k, generator=g) * 0.02
+            q, sc = mxfp8_quantize_device(w.to(dev), code_pitch(k))
+            qs.append(q)
+            scs.append(sc)
+        return torch.stack(qs), torch.stack(scs)
+
+    wg = weights(I, H)
+    wu = weights(I, H)
+    wd = weights(H, I)
+    return dict(tokens_per_expert=counts.to(dev), row_token=row_token.to(dev), x_q=x_q, x_sc=x_sc, w_gate_q=wg[0],
+                w_gate_sc=wg[1], w_up_q=wu[0], w_up_sc=wu[1], w_down_q=wd[0], w_down_sc=wd[1])
+
+
+def cpu_baseline(inp, sample_tokens=1024, reps=3):
+    """The oracle on the host cores, first `sample_tokens` tokens of the same inputs."""
+    import numpy as np
+    import torch
+    from oracle import moe_ffn
+    from pipelink_amd.host import mok_inputs
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(0)
+    logits = torch.randn(T, E, generator=g)[:sample_tokens]
+    counts, row_token = mok_inputs.route(logits, TOPK)
+    host = {k: v.cpu() for k, v in inp.items()}
+    args = dict(x_q=host["x_q"][:sample_tokens, :H], x_sc=host["x_sc"][:sample_tokens],
+                wg_q=host["w_gate_q"][:, :, :H], wg_sc=host["w_gate_sc"], wu_q=host["w_up_q"][:, :, :H],
+                wu_sc=host["w_up_sc"], wd_q=host["w_down_q"][:, :, :I], wd_sc=host["w_down_sc"], counts=counts,
+                row_token=row_token)
+    times = []
+    for rep in range(reps + 1):
+        t0 = time.perf_counter()
+        moe_ffn.moe_ffn_forward_torch(**args)
+        if rep:
+            times.append(time.perf_counter() - t0)
+    sec = statistics.median(times)
+    flops = FLOPS_TOTAL * sample_tokens / T
+    return {"value": round(flops / sec / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"first {sample_tokens} of {T} tokens (all {E} experts' weights dequantised inside the timed "
+                      f"region), median of {reps} runs after 1 warm-up, {sec * 1e3:.0f} ms per forward, "
+                      f"torch {torch.__version__} fp32"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-pair", action="store_true", help="skip the linked vs one-unit paired timing")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU's share of the routed-expert FFN; --gpus must be 1",
+              file=sys.stderr)
+        return 2
+
+    import torch
+    from pipelink_amd.host.backend import HipBackend
+    from pipelink_amd.host.mok import MoKSession, code_pitch, scale_pitch
+    from pipelink_amd.stages.mok import build as mok_build
+
+    paths = mok_build.images()  # raises if the HIP images are missing: there is no fallback path
+    dev = torch.device("cuda:0")
+    inp = make_inputs(dev)
+    rows = T * TOPK
+    hq = torch.zeros((rows, code_pitch(I)), dtype=torch.uint8, device=dev)
+    hsc = torch.zeros((rows, scale_pitch(I)), dtype=torch.uint8, device=dev)
+    y = torch.full((rows, H), float("nan"), dtype=torch.bfloat16, device=dev)
+    link_json = json.loads(paths["link_json"].read_text())
+    linked = MoKSession(paths["linked"].read_bytes(), link_json)
+    control = MoKSession(paths["one_unit"].read_bytes(), link_json)
+    prob = linked.problem(hidden_q=hq, hidden_sc=hsc, y=y, **inp)
+    stream = torch.cuda.current_stream().cuda_stream
+    be = HipBackend(0, stream)
+
+    for _ in range(args.warmup):
+        linked.forward(prob)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        linked.forward(prob)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    def event_ms(sess, which, n):
+        e0, e1 = be.event_create(), be.event_create()
+        be.event_record(e0)
+        for _ in range(n):
+            sess.forward(prob, which=which)
+        be.event_record(e1)
+        be.event_synchronize(e1)
+        ms = be.event_elapsed_time(e0, e1) / n
+        be.event_destroy(e0)
+        be.event_destroy(e1)
+        return ms
+
+    n = max(args.steps, 10)
+    ms_gate_up = event_ms(linked, 1, n)
+    ms_down = event_ms(linked, 2, n)
+
+    pair = None
+    if not args.no_pair:
+        # 8 blocks in the orders ABBA BAAB BAAB ABBA BAAB ABBA ABBA BAAB (A = linked, B = one-unit)
+        orders = ["ABBA", "BAAB", "BAAB", "ABBA", "BAAB", "ABBA", "ABBA", "BAAB"]
+        batch = max(5, int(16.0 / max(ms_per_step, 1e-3)))
+        for s in (linked, control):
+            for _ in range(8):
+                s.forward(prob)
+        ratios = []
+        for order in orders:
+            t = {"A": 0.0, "B": 0.0}
+            for c in order:
+                t[c] += event_ms(linked if c == "A" else control, 0, batch)
+            ratios.append(t["B"] / t["A"])  # > 1: linked faster
+        pair = {"speed_ratio": round(statistics.median(ratios), 5), "blocks": [round(r, 5) for r in ratios],
+                "batch": batch, "definition": "one-unit time / linked time, median of 8 ABBA/BAAB blocks"}
+
+    out = {
+        "metric": "MXFP8 MoE grouped-GEMM TFLOP/s (% MFMA peak); linked/one-unit speed ratio",
+        "value": round(FLOPS_TOTAL / (ms_per_step * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3 (MXFP8, fp32 accumulate)",
+        "data": "synthetic",
+        "config": {"workload": "configs[2]: MXFP8 MoE expert FFN forward", "tokens": T, "d_model": H, "d_ff": I,
+                   "experts": E, "top_k": TOPK, "routed_rows": rows, "image": "linked",
+                   "pct_of_fp8_mfma_peak": round(FLOPS_TOTAL / (ms_per_step * 1e-3) / 1e12 / PEAK_FP8_TFLOPS * 100, 2),
+                   "ms_per_token": round(ms_per_step / T, 7)},
+        "roofline": {"bound": "mfma", "kernel": "pipelink_kernel (gate/up pass: grouped GEMM + SwiGLU + requant)",
+                     "achieved": round(FLOPS_GATE_UP / (ms_gate_up * 1e-3) / 1e12, 2), "peak": PEAK_FP8_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(FLOPS_GATE_UP / (ms_gate_up * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4),
+                     "traffic": None, "launch_ms": round(ms_gate_up, 4),
+                     "down_pass": {"achieved": round(FLOPS_DOWN / (ms_down * 1e-3) / 1e12, 2), "launch_ms": round(ms_down, 4)}},
+        "linked_over_one_unit": pair,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(inp)
+    print(json.dumps(out))
+    linked.close()
+    control.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

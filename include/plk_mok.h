@@ -10,7 +10,9 @@
  * and the down pass on the caller's stream.  All tensor arguments are device addresses
  * owned by the caller; nothing is allocated per call.
  *
- * Operand layouts (all row-major):
+ * Operand layouts (all row-major; a code row may be padded to a pitch ld_q >= K, a multiple
+ * of 16 -- a pitch that is a multiple of 128 makes every ring-slot row one aligned cache
+ * line, which is what the loader is fastest on):
  *   x_q [T,H] e4m3, x_sc [T,ld_sc_h] e8m0 (one byte per 32 elements of H; ld_sc_h % 4 == 0)
  *   w_gate_q / w_up_q [E,I,H], scales [E,I,ld_sc_h];  w_down_q [E,H,I], scales [E,H,ld_sc_i]
  *   tokens_per_expert [E] i32, row_token [R] i32 (routed row -> token; 0 = rows are tokens)
@@ -46,6 +48,8 @@ typedef struct plk_mok_problem {
   int32_t routed_rows;   /* R = sum(tokens_per_expert) */
   int32_t ld_sc_h;       /* scale row pitch for K = H operands */
   int32_t ld_sc_i;       /* scale row pitch for K = I operands */
+  int32_t ld_q_h;        /* code row pitch in bytes for K = H operands (x, w_gate, w_up); 0 = H */
+  int32_t ld_q_i;        /* code row pitch in bytes for K = I operands (hidden, w_down); 0 = I */
   float swiglu_limit;
   int32_t reserved;
   uint64_t x_q, x_sc, row_token, tokens_per_expert;
@@ -63,9 +67,10 @@ int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass,
 
 /* MXFP8 block quantiser on the device (what ops.mxfp8_quantize does for the reference's
  * harness, campaigns/mok/host/mok_port_host.py:122): src is fp32 (src_is_bf16 = 0) or bf16
- * [rows, k], dst_q [rows, k] e4m3, dst_sc [rows, ld_sc] e8m0 (padding bytes zeroed). */
-int plk_mxfp8_quantize(uint64_t src, int src_is_bf16, int64_t rows, int32_t k, uint64_t dst_q, uint64_t dst_sc,
-                       int32_t ld_sc, void* stream);
+ * [rows, k], dst_q [rows, ld_q] e4m3 (ld_q >= k; pad bytes untouched), dst_sc [rows, ld_sc] e8m0
+ * (padding bytes zeroed). */
+int plk_mxfp8_quantize(uint64_t src, int src_is_bf16, int64_t rows, int32_t k, uint64_t dst_q, int32_t ld_q,
+                       uint64_t dst_sc, int32_t ld_sc, void* stream);
 
 #ifdef __cplusplus
 }

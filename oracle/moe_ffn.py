@@ -136,3 +136,51 @@ def rel_frobenius(got: np.ndarray, ref: np.ndarray) -> float:
     r = np.asarray(ref, dtype=np.float64)
     den = float(np.sqrt(np.sum(r * r)))
     return float(np.sqrt(np.sum((g - r) ** 2)) / den) if den else float(np.sqrt(np.sum(g * g)))
+
+
+# ---- the same pipeline in torch ops (multi-threaded; what bench.py times as the CPU baseline) ----
+def _deq_torch(q: torch.Tensor, sc: torch.Tensor) -> torch.Tensor:
+    k = q.shape[-1]
+    nb = k // mxfp8.MX_BLOCK
+    vals = q.contiguous().view(torch.float8_e4m3fn).float().reshape(q.shape[:-1] + (nb, mxfp8.MX_BLOCK))
+    scale = ((sc[..., :nb].to(torch.int32)) << 23).view(torch.float32)  # 2**(b-127) for 1 <= b <= 254
+    scale = torch.where(sc[..., :nb] == 0, torch.full_like(scale, 2.0 ** -127), scale)
+    return (vals * scale.unsqueeze(-1)).reshape(q.shape)
+
+
+def _quant_torch(x: torch.Tensor):
+    nb = x.shape[-1] // mxfp8.MX_BLOCK
+    blk = x.reshape(x.shape[:-1] + (nb, mxfp8.MX_BLOCK))
+    amax = blk.abs().amax(dim=-1)
+    b = (((amax.view(torch.int32) >> 23) & 0xFF) - 8).clamp_(0, 254)
+    inv = ((254 - b) << 23).view(torch.float32)
+    codes = (blk * inv.unsqueeze(-1)).clamp_(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
+    return codes.reshape(x.shape), b.to(torch.uint8)
+
+
+def moe_ffn_forward_torch(x_q, x_sc, wg_q, wg_sc, wu_q, wu_sc, wd_q, wd_sc, counts, row_token,
+                          limit: float | None = 7.0, alpha: float = SWIGLU_ALPHA) -> torch.Tensor:
+    """Same arithmetic as ``moe_ffn_forward`` with torch kernels; returns y as bf16 [R, H]."""
+    a = _deq_torch(x_q, x_sc)[row_token.long()]
+    rows = a.shape[0]
+    hidden = torch.empty((rows, wg_q.shape[1]), dtype=torch.float32)
+    off = 0
+    for e, c in enumerate(counts.tolist()):
+        if c:
+            ae = a[off:off + c]
+            g = ae @ _deq_torch(wg_q[e], wg_sc[e]).t()
+            u = ae @ _deq_torch(wu_q[e], wu_sc[e]).t()
+            if limit is not None:
+                g = g.clamp(max=limit)
+                u = u.clamp(min=-limit, max=limit)
+            hidden[off:off + c] = ((u + 1.0) * (g * torch.sigmoid(alpha * g))).to(torch.bfloat16).float()
+        off += c
+    hq, hb = _quant_torch(hidden)
+    hd = _deq_torch(hq, hb)
+    y = torch.empty((rows, wd_q.shape[1]), dtype=torch.float32)
+    off = 0
+    for e, c in enumerate(counts.tolist()):
+        if c:
+            y[off:off + c] = hd[off:off + c] @ _deq_torch(wd_q[e], wd_sc[e]).t()
+        off += c
+    return y.to(torch.bfloat16)

@@ -6,6 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -39,6 +40,8 @@ static int check_problem(const plk_mok_problem* p) {
     return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: hidden and intermediate must be positive multiples of 64");
   if (p->ld_sc_h % 4 || p->ld_sc_i % 4 || p->ld_sc_h * 32 < p->hidden || p->ld_sc_i * 32 < p->intermediate)
     return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: scale pitch must be a multiple of 4 covering K/32 blocks");
+  if ((p->ld_q_h && (p->ld_q_h < p->hidden || p->ld_q_h % 16)) || (p->ld_q_i && (p->ld_q_i < p->intermediate || p->ld_q_i % 16)))
+    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: code row pitch must be a multiple of 16 and at least K");
   if (p->num_tokens < 0 || p->routed_rows < 0)
     return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: negative row count");
   if (p->routed_rows && (!p->x_q || !p->x_sc || !p->tokens_per_expert || !p->w_gate_q || !p->w_gate_sc ||
@@ -48,15 +51,15 @@ static int check_problem(const plk_mok_problem* p) {
   return PLK_OK;
 }
 
-static MokMxView view(uint64_t q, uint64_t sc, int64_t rows, int k, int ld_sc, bool per_expert) {
+static MokMxView view(uint64_t q, uint64_t sc, int64_t rows, int k, int ld_q, int ld_sc, bool per_expert) {
   MokMxView v{};
   v.q = (const uint8_t*)(uintptr_t)q;
   v.sc = (const uint8_t*)(uintptr_t)sc;
   v.rows = (int32_t)rows;
   v.k = k;
-  v.ld_q = k;
+  v.ld_q = ld_q;
   v.ld_sc = ld_sc;
-  v.expert_pitch_q = per_expert ? rows * (int64_t)k : 0;
+  v.expert_pitch_q = per_expert ? rows * (int64_t)ld_q : 0;
   v.expert_pitch_sc = per_expert ? rows * (int64_t)ld_sc : 0;
   return v;
 }
@@ -123,11 +126,12 @@ int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass,
   fw.num_col_tiles = pass == 1 ? (I + TILE_W / 2 - 1) / (TILE_W / 2) : (H + TILE_W - 1) / TILE_W;
 
   MokGemmResidue g{};
-  g.x = view(p->x_q, p->x_sc, p->num_tokens, H, p->ld_sc_h, false);
-  g.hidden = view(p->hidden_q, p->hidden_sc, p->routed_rows, I, p->ld_sc_i, false);
-  g.w_gate = view(p->w_gate_q, p->w_gate_sc, I, H, p->ld_sc_h, true);
-  g.w_up = view(p->w_up_q, p->w_up_sc, I, H, p->ld_sc_h, true);
-  g.w_down = view(p->w_down_q, p->w_down_sc, H, I, p->ld_sc_i, true);
+  const int ldh = p->ld_q_h ? p->ld_q_h : H, ldi = p->ld_q_i ? p->ld_q_i : I;
+  g.x = view(p->x_q, p->x_sc, p->num_tokens, H, ldh, p->ld_sc_h, false);
+  g.hidden = view(p->hidden_q, p->hidden_sc, p->routed_rows, I, ldi, p->ld_sc_i, false);
+  g.w_gate = view(p->w_gate_q, p->w_gate_sc, I, H, ldh, p->ld_sc_h, true);
+  g.w_up = view(p->w_up_q, p->w_up_sc, I, H, ldh, p->ld_sc_h, true);
+  g.w_down = view(p->w_down_q, p->w_down_sc, H, I, ldi, p->ld_sc_i, true);
   g.row_token = (const int32_t*)(uintptr_t)p->row_token;
   g.y = (uint16_t*)(uintptr_t)p->y;
   g.ld_y = H;
@@ -137,7 +141,7 @@ int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass,
   a.hidden_sc = (uint8_t*)(uintptr_t)p->hidden_sc;
   a.rows = p->routed_rows;
   a.cols = I;
-  a.ld_q = I;
+  a.ld_q = ldi;
   a.ld_sc = p->ld_sc_i;
   a.swiglu_limit = p->swiglu_limit;
 
@@ -158,6 +162,7 @@ int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass,
   const int64_t max_tiles = max_row_tiles * fw.num_col_tiles;
   int64_t wgs = (int64_t)s->compute_units * s->link.workgroups_per_cu;
   if (wgs > max_tiles) wgs = max_tiles;
+  if (const char* dbg = getenv("PLK_MOK_DEBUG_GRID")) wgs = atoll(dbg);
   wgs = (wgs + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
   const uint32_t grid[3] = {(uint32_t)wgs, 1, 1};
   const uint32_t block[3] = {s->link.threads, 1, 1};
@@ -178,8 +183,8 @@ int plk_mok_forward(plk_mok_session* s, const plk_mok_problem* p, void* stream) 
 // e4m3_rne(clamp(v * 2^(127 - byte), +-448)).
 template <bool BF16>
 __global__ void __launch_bounds__(256) mxfp8_quantize_kernel(const void* __restrict__ src, int64_t rows, int k,
-                                                             uint8_t* __restrict__ dq, uint8_t* __restrict__ dsc,
-                                                             int ld_sc) {
+                                                             uint8_t* __restrict__ dq, int ld_q,
+                                                             uint8_t* __restrict__ dsc, int ld_sc) {
   const int blocks_per_row = k / 32;
   const int64_t nblocks = rows * (int64_t)blocks_per_row;
   const int sub = threadIdx.x & 7;
@@ -210,7 +215,7 @@ __global__ void __launch_bounds__(256) mxfp8_quantize_kernel(const void* __restr
     int pk = 0;
     pk = __builtin_amdgcn_cvt_pk_fp8_f32(s[0], s[1], pk, false);
     pk = __builtin_amdgcn_cvt_pk_fp8_f32(s[2], s[3], pk, true);
-    *reinterpret_cast<uint32_t*>(dq + off) = (uint32_t)pk;
+    *reinterpret_cast<uint32_t*>(dq + row * (int64_t)ld_q + cb * 32 + sub * 4) = (uint32_t)pk;
     if (sub == 0) dsc[row * ld_sc + cb] = (uint8_t)e;
     // zero the pad bytes of the scale row once per row
     if (cb == 0 && sub == 1)
@@ -219,9 +224,10 @@ __global__ void __launch_bounds__(256) mxfp8_quantize_kernel(const void* __restr
 }
 
 extern "C" int plk_mxfp8_quantize(uint64_t src, int src_is_bf16, int64_t rows, int32_t k, uint64_t dst_q,
-                                  uint64_t dst_sc, int32_t ld_sc, void* stream) {
-  if (rows < 0 || k <= 0 || k % 32 || ld_sc * 32 < k)
-    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mxfp8_quantize: k must be a positive multiple of 32 covered by ld_sc");
+                                  int32_t ld_q, uint64_t dst_sc, int32_t ld_sc, void* stream) {
+  if (rows < 0 || k <= 0 || k % 32 || ld_sc * 32 < k || ld_q < k || ld_q % 4)
+    return plk_hip_set_error(PLK_E_ARGUMENT,
+                             "plk_mxfp8_quantize: k must be a positive multiple of 32 covered by ld_sc and ld_q");
   if (rows == 0) return PLK_OK;
   if (!src || !dst_q || !dst_sc) return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mxfp8_quantize: null device address");
   const int64_t nblocks = rows * (int64_t)(k / 32);
@@ -229,10 +235,10 @@ extern "C" int plk_mxfp8_quantize(uint64_t src, int src_is_bf16, int64_t rows, i
   if (grid > 65536) grid = 65536;
   if (src_is_bf16)
     mxfp8_quantize_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>(
-        (const void*)(uintptr_t)src, rows, k, (uint8_t*)(uintptr_t)dst_q, (uint8_t*)(uintptr_t)dst_sc, ld_sc);
+        (const void*)(uintptr_t)src, rows, k, (uint8_t*)(uintptr_t)dst_q, ld_q, (uint8_t*)(uintptr_t)dst_sc, ld_sc);
   else
     mxfp8_quantize_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>(
-        (const void*)(uintptr_t)src, rows, k, (uint8_t*)(uintptr_t)dst_q, (uint8_t*)(uintptr_t)dst_sc, ld_sc);
+        (const void*)(uintptr_t)src, rows, k, (uint8_t*)(uintptr_t)dst_q, ld_q, (uint8_t*)(uintptr_t)dst_sc, ld_sc);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return plk_hip_set_error(PLK_E_RESOURCE, hipGetErrorString(e));
   return PLK_OK;

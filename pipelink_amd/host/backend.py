@@ -38,7 +38,7 @@ class MokLinkInfo(ctypes.Structure):
 class MokProblem(ctypes.Structure):
     _fields_ = [("struct_bytes", c_uint32), ("num_tokens", c_int32), ("hidden", c_int32), ("intermediate", c_int32),
                 ("num_experts", c_int32), ("routed_rows", c_int32), ("ld_sc_h", c_int32), ("ld_sc_i", c_int32),
-                ("swiglu_limit", c_float), ("reserved", c_int32)] + \
+                ("ld_q_h", c_int32), ("ld_q_i", c_int32), ("swiglu_limit", c_float), ("reserved", c_int32)] + \
                [(n, c_uint64) for n in ("x_q", "x_sc", "row_token", "tokens_per_expert", "w_gate_q", "w_gate_sc",
                                         "w_up_q", "w_up_sc", "w_down_q", "w_down_sc", "hidden_q", "hidden_sc", "y")]
 
@@ -71,7 +71,7 @@ SIGNATURES = {
     "plk_mok_session_destroy": (c_int, [c_void_p]),
     "plk_mok_forward": (c_int, [c_void_p, POINTER(MokProblem), c_void_p]),
     "plk_mok_forward_pass": (c_int, [c_void_p, POINTER(MokProblem), c_int, c_void_p]),
-    "plk_mxfp8_quantize": (c_int, [c_uint64, c_int, c_int64, c_int32, c_uint64, c_uint64, c_int32, c_void_p]),
+    "plk_mxfp8_quantize": (c_int, [c_uint64, c_int, c_int64, c_int32, c_uint64, c_int32, c_uint64, c_int32, c_void_p]),
 }
 
 _lib = None

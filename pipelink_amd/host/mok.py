@@ -66,21 +66,24 @@ class MoKSession:
                             w_down_sc=w_down_sc, hidden_q=hidden_q, hidden_sc=hidden_sc, y=y).items():
             if not t.is_cuda or not t.is_contiguous():
                 raise PlkError(3, f"{name} must be a contiguous device tensor")
-        t_rows, h = x_q.shape
-        e, i, h2 = w_gate_q.shape
-        r = y.shape[0]
-        if h2 != h or tuple(w_up_q.shape) != (e, i, h) or tuple(w_down_q.shape) != (e, h, i):
-            raise PlkError(3, "weight shapes disagree with x")
-        if tuple(hidden_q.shape) != (r, i) or y.shape[1] != h or y.dtype != torch.bfloat16:
+        # code tensors may carry a padded last dimension (row pitch); the logical K comes from y / w_down
+        t_rows, ldh = x_q.shape
+        r, h = y.shape
+        e, i, ldh2 = w_gate_q.shape
+        ldi_q = hidden_q.shape[1]
+        if ldh2 != ldh or tuple(w_up_q.shape) != (e, i, ldh) or tuple(w_down_q.shape) != (e, h, ldi_q):
+            raise PlkError(3, "weight shapes disagree with x / hidden")
+        if hidden_q.shape[0] != r or y.dtype != torch.bfloat16 or ldh < h or ldi_q < i:
             raise PlkError(3, "hidden_q / y shapes disagree")
-        ldh, ldi = scale_pitch(h), scale_pitch(i)
-        if x_sc.shape[1] != ldh or w_gate_sc.shape[2] != ldh or w_up_sc.shape[2] != ldh or \
-                w_down_sc.shape[2] != ldi or hidden_sc.shape[1] != ldi:
+        ldsh, ldsi = scale_pitch(h), scale_pitch(i)
+        if x_sc.shape[1] != ldsh or w_gate_sc.shape[2] != ldsh or w_up_sc.shape[2] != ldsh or \
+                w_down_sc.shape[2] != ldsi or hidden_sc.shape[1] != ldsi:
             raise PlkError(3, "scale pitch must be K/32 rounded up to a multiple of 4")
         if tokens_per_expert.dtype != torch.int32 or (row_token is not None and row_token.dtype != torch.int32):
             raise PlkError(3, "tokens_per_expert and row_token must be int32")
         return MokProblem(struct_bytes=sizeof(MokProblem), num_tokens=t_rows, hidden=h, intermediate=i, num_experts=e,
-                          routed_rows=r, ld_sc_h=ldh, ld_sc_i=ldi, swiglu_limit=swiglu_limit,
+                          routed_rows=r, ld_sc_h=ldsh, ld_sc_i=ldsi, ld_q_h=ldh, ld_q_i=ldi_q,
+                          swiglu_limit=swiglu_limit,
                           x_q=x_q.data_ptr(), x_sc=x_sc.data_ptr(),
                           row_token=0 if row_token is None else row_token.data_ptr(),
                           tokens_per_expert=tokens_per_expert.data_ptr(),
@@ -97,15 +100,24 @@ class MoKSession:
             check(self.lib, self.lib.plk_mok_forward_pass(self._handle, byref(problem), which, s))
 
 
-def mxfp8_quantize_device(src: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
-    """Quantise a 2-D fp32 or bf16 device tensor along its last axis on the GPU."""
+def code_pitch(k: int, align: int = 128) -> int:
+    """Row pitch in bytes of an e4m3 operand whose rows start on `align`-byte boundaries."""
+    return (k + align - 1) // align * align
+
+
+def mxfp8_quantize_device(src: torch.Tensor, pitch: int | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Quantise a 2-D fp32 or bf16 device tensor along its last axis on the GPU.
+
+    ``pitch`` pads every code row to that many bytes (pad bytes are zero)."""
     if not src.is_cuda or not src.is_contiguous() or src.dim() != 2 or src.dtype not in (torch.float32, torch.bfloat16):
         raise PlkError(3, "src must be a contiguous 2-D fp32/bf16 device tensor")
     rows, k = src.shape
     ld = scale_pitch(k)
-    q = torch.empty((rows, k), dtype=torch.uint8, device=src.device)
+    pitch = k if pitch is None else pitch
+    q = torch.empty((rows, pitch), dtype=torch.uint8, device=src.device) if pitch == k else \
+        torch.zeros((rows, pitch), dtype=torch.uint8, device=src.device)
     sc = torch.empty((rows, ld), dtype=torch.uint8, device=src.device)
     lib = load_library()
-    check(lib, lib.plk_mxfp8_quantize(src.data_ptr(), int(src.dtype == torch.bfloat16), rows, k, q.data_ptr(),
+    check(lib, lib.plk_mxfp8_quantize(src.data_ptr(), int(src.dtype == torch.bfloat16), rows, k, q.data_ptr(), pitch,
                                       sc.data_ptr(), ld, c_void_p(torch.cuda.current_stream().cuda_stream)))
     return q, sc

@@ -1,0 +1,160 @@
+// Authoring annotations of a PipeLink stage source for gfx950.
+//
+// In the device compile (hipcc) every PL_* macro expands to nothing.  With -DPIPELINK_EMIT the
+// stage source is compiled as a host C++17 program instead (the device code is fenced off with
+// `#ifndef PIPELINK_EMIT`): the macros become static registrations whose records -- evaluated
+// with the real sizeof/alignof of the stage's own types -- are printed as one JSON object by
+// pl::emit_main(), from which `pipec pack` assembles manifest.json.
+//
+// Same division of labour and macro names as the reference's
+// pipec/src/pipec2/pack/include/pipelink/stage.hpp:1413-1477 (registrations) / :1488-1524
+// (no-ops) and pack/runner.cpp; the record set is the subset the gfx950 backend consumes
+// (stage, params, roles, exports, call seams, claims, counter and ring endpoints, variants,
+// topology, facts).
+#ifndef PIPELINK_STAGE_HPP
+#define PIPELINK_STAGE_HPP
+
+#ifdef PIPELINK_EMIT
+
+#include <cstdio>
+#include <initializer_list>
+#include <string>
+#include <utility>
+#include <vector>
+
+namespace pl {
+
+inline std::vector<std::pair<std::string, std::string>>& registry() {
+  static std::vector<std::pair<std::string, std::string>> r;  // (section, json object)
+  return r;
+}
+
+inline std::string quote(const std::string& s) {
+  std::string out = "\"";
+  for (char c : s) {
+    if (c == '"' || c == '\\') { out += '\\'; out += c; }
+    else if (c == '\n') out += "\\n";
+    else out += c;
+  }
+  return out + "\"";
+}
+
+struct reg {
+  reg(const char* section, const std::string& json) { registry().emplace_back(section, json); }
+};
+
+inline std::string num(long long v) { return std::to_string(v); }
+
+struct kv { const char* handle; long long value; };
+
+inline std::string keyset(std::initializer_list<kv> key) {
+  std::string out = "{";
+  bool first = true;
+  for (const kv& k : key) {
+    if (!first) out += ",";
+    first = false;
+    out += quote(k.handle) + ":" + num(k.value);
+  }
+  return out + "}";
+}
+
+inline std::string strlist(std::initializer_list<const char*> items) {
+  std::string out = "[";
+  bool first = true;
+  for (const char* s : items) {
+    if (!first) out += ",";
+    first = false;
+    out += quote(s);
+  }
+  return out + "]";
+}
+
+inline int emit_main() {
+  // {"section": [records...], ...} with sections in first-use order
+  std::vector<std::string> sections;
+  for (auto& e : registry()) {
+    bool seen = false;
+    for (auto& s : sections) seen = seen || s == e.first;
+    if (!seen) sections.push_back(e.first);
+  }
+  std::printf("{");
+  for (size_t i = 0; i < sections.size(); ++i) {
+    std::printf("%s%s:[", i ? "," : "", quote(sections[i]).c_str());
+    bool first = true;
+    for (auto& e : registry())
+      if (e.first == sections[i]) {
+        std::printf("%s%s", first ? "" : ",", e.second.c_str());
+        first = false;
+      }
+    std::printf("]");
+  }
+  std::printf("}\n");
+  return 0;
+}
+
+}  // namespace pl
+
+#define PL_CAT2(a, b) a##b
+#define PL_CAT(a, b) PL_CAT2(a, b)
+#define PL_REG(section, json) static const ::pl::reg PL_CAT(pl_reg_, __COUNTER__)(section, json)
+
+#define PL_STAGE(id, version) PL_REG("stage", "{\"id\":" + ::pl::quote(id) + ",\"version\":" + ::pl::quote(version) + "}")
+#define PL_PARAMS(T) \
+  PL_REG("params", "{\"type\":" + ::pl::quote(#T) + ",\"bytes\":" + ::pl::num(sizeof(T)) + ",\"align\":" + ::pl::num(alignof(T)) + "}")
+#define PL_NO_PARAMS() PL_REG("params", "{\"type\":\"void\",\"bytes\":0,\"align\":1}")
+#define PL_ROLE(name, fn, warps) \
+  PL_REG("roles", "{\"name\":" + ::pl::quote(#name) + ",\"entry\":" + ::pl::quote(#fn) + ",\"warps\":" + ::pl::num(warps) + "}")
+// an exported device function: `decl` is its declaration text, identity-bearing for the call seam
+#define PL_EXPORT(name, symbol, decl) \
+  PL_REG("exports", "{\"name\":" + ::pl::quote(#name) + ",\"symbol\":" + ::pl::quote(#symbol) + ",\"decl\":" + ::pl::quote(decl) + "}")
+// this stage calls export `export_name` of whoever consumes channel `channel` through the
+// link-generated trampoline pipelink_call_<channel>; `decl` declares that trampoline
+#define PL_CALL(channel, export_name, decl) \
+  PL_REG("calls", "{\"channel\":" + ::pl::quote(#channel) + ",\"direction\":\"produce\",\"export\":" + ::pl::quote(export_name) + ",\"decl\":" + ::pl::quote(decl) + "}")
+// this stage provides export `export_name` on channel `channel`
+#define PL_SERVE(channel, export_name) \
+  PL_REG("calls", "{\"channel\":" + ::pl::quote(#channel) + ",\"direction\":\"consume\",\"export\":" + ::pl::quote(export_name) + "}")
+#define PL_CLAIM(handle, domain, extent, align, lifetime) \
+  PL_REG("claims", "{\"handle\":" + ::pl::quote(handle) + ",\"domain\":" + ::pl::quote(domain) + ",\"extent\":{\"const\":" + ::pl::num(extent) + ",\"per\":{}},\"align\":" + ::pl::num(align) + ",\"lifetime\":" + ::pl::quote(lifetime) + "}")
+// extent = base + per * value(depth_handle): an LDS ring whose depth is bound at link time
+#define PL_CLAIM_RING(handle, domain, base, depth_handle, per, align, lifetime) \
+  PL_REG("claims", "{\"handle\":" + ::pl::quote(handle) + ",\"domain\":" + ::pl::quote(domain) + ",\"extent\":{\"const\":" + ::pl::num(base) + ",\"per\":{" + ::pl::quote(depth_handle) + ":" + ::pl::num(per) + "}},\"align\":" + ::pl::num(align) + ",\"lifetime\":" + ::pl::quote(lifetime) + "}")
+#define PL_VARIANT(index, ...) \
+  PL_REG("variants", "{\"index\":" + ::pl::num(index) + ",\"key\":" + ::pl::keyset(__VA_ARGS__) + "}")
+#define PL_TOPOLOGY(persistent, scheduler) \
+  PL_REG("topology", std::string("{\"persistent\":") + ((persistent) ? "true" : "false") + ",\"scheduler\":" + ::pl::quote(scheduler) + "}")
+// a global-memory counter channel: release add on the producing side, acquire load on the other
+#define PL_COUNTER(name, direction, slot_handle, exports) \
+  PL_REG("counters", "{\"name\":" + ::pl::quote(#name) + ",\"direction\":" + ::pl::quote(direction) + ",\"slot\":" + ::pl::quote(slot_handle) + ",\"exports\":" + ::pl::strlist(exports) + "}")
+// a published geometry fact of this owner (reaches other owners only through the link)
+#define PL_FACT(name, value) PL_REG("facts", "{\"name\":" + ::pl::quote(name) + ",\"value\":" + ::pl::num(value) + "}")
+// a header whose declarations cross a call seam (task records, fragment types): its text
+// travels in the package and the linker puts it in front of the generated trampolines
+#define PL_PRELUDE(path) PL_REG("preludes", ::pl::quote(path))
+// handles this stage reads through `extern "C" __device__ int <handle>()`
+#define PL_USES(handle) PL_REG("uses", ::pl::quote(handle))
+
+#define PL_EMIT_MAIN() \
+  int main() { return ::pl::emit_main(); }
+
+#else  // device compile: annotations vanish
+
+#define PL_STAGE(id, version)
+#define PL_PARAMS(T)
+#define PL_NO_PARAMS()
+#define PL_ROLE(name, fn, warps)
+#define PL_EXPORT(name, symbol, decl)
+#define PL_CALL(channel, export_name, decl)
+#define PL_SERVE(channel, export_name)
+#define PL_CLAIM(handle, domain, extent, align, lifetime)
+#define PL_CLAIM_RING(handle, domain, base, depth_handle, per, align, lifetime)
+#define PL_VARIANT(index, ...)
+#define PL_TOPOLOGY(persistent, scheduler)
+#define PL_COUNTER(name, direction, slot_handle, exports)
+#define PL_FACT(name, value)
+#define PL_USES(handle)
+#define PL_PRELUDE(path)
+#define PL_EMIT_MAIN()
+
+#endif
+#endif

@@ -10,6 +10,8 @@
 // The body only uses the placement contract of mok::AccFrag (which routed row and column
 // a (fragment, register, lane) triple is); it does not care whether the GEMM owner kept
 // the accumulator in AGPRs, VGPRs or LDS.
+#include <pipelink/stage.hpp>
+#ifndef PIPELINK_EMIT
 #include "../include/mok_device.hpp"
 
 extern "C" __device__ int pipelink_mok_clamp();  // link-time variant: 1 = clamp to +-limit
@@ -92,3 +94,23 @@ extern "C" __device__ void mok_act_fwd(const void* view, const MokActTask* task,
   else
     mok_act_owner::forward<false>(p, *task, *acc);
 }
+#else  // PIPELINK_EMIT: host-evaluated annotations only
+#include "../include/mok_abi.h"
+#endif
+
+PL_STAGE("mok.act", "0.1.0-gptoss");
+PL_PARAMS(MokActResidue);
+PL_TOPOLOGY(true, "static");
+// clamp on/off is a link-time variant (campaigns/mok/port/act_gptoss/act.cu:246-249)
+PL_VARIANT(0, {{"pipelink_mok_clamp", 0}});
+PL_VARIANT(1, {{"pipelink_mok_clamp", 1}});
+PL_EXPORT(mok_act_init, mok_act_init, "extern \"C\" __device__ void mok_act_init(const void* view);");
+PL_EXPORT(mok_act_fwd, mok_act_fwd,
+          "extern \"C\" __device__ void mok_act_fwd(const void* view, const MokActTask* task, "
+          "const MokCounters* counters, uint32_t* phase, const mok::AccFrag* acc);");
+PL_SERVE(act_init, "mok_act_init");
+PL_SERVE(act_fwd, "mok_act_fwd");
+PL_USES("pipelink_mok_clamp");
+PL_PRELUDE("../include/mok_abi.h");
+PL_PRELUDE("../include/mok_device.hpp");
+PL_EMIT_MAIN()

@@ -10,6 +10,8 @@
 // innermost, so workgroups that run at the same time share one weight tile; the tile
 // range is split in 8 contiguous chunks, one per XCD (workgroup id % 8), so each L2 sees
 // a contiguous run of experts.
+#include <pipelink/stage.hpp>
+#ifndef PIPELINK_EMIT
 #include "../include/mok_device.hpp"
 
 extern "C" __device__ int pipelink_mok_fw_sched();  // byte offset of the schedule table in dynamic LDS
@@ -87,3 +89,27 @@ extern "C" __device__ void mok_framework_worker(const void* params, unsigned var
     }
   }
 }
+#else  // PIPELINK_EMIT: host-evaluated annotations only
+#include "../include/mok_abi.h"
+#endif
+
+PL_STAGE("mok.framework", "0.1.0");
+PL_PARAMS(MokFrameworkParams);
+PL_ROLE(worker, mok_framework_worker, 8);
+PL_TOPOLOGY(true, "static");
+PL_VARIANT(0, {});
+PL_CALL(gemm_init, "mok_gemm_init", "extern \"C\" __device__ void pipelink_call_gemm_init(const void* view);");
+PL_CALL(act_init, "mok_act_init", "extern \"C\" __device__ void pipelink_call_act_init(const void* view);");
+PL_CALL(gemm_fwd, "mok_gemm_fwd",
+        "extern \"C\" __device__ void pipelink_call_gemm_fwd(const void* view, const MokGemmTask* task, "
+        "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc);");
+PL_CALL(act_fwd, "mok_act_fwd",
+        "extern \"C\" __device__ void pipelink_call_act_fwd(const void* view, const MokActTask* task, "
+        "const MokCounters* counters, uint32_t* phase, const mok::AccFrag* acc);");
+// schedule table: exclusive prefix sums of rows and row tiles for up to 256 experts
+PL_CLAIM("pipelink_mok_fw_sched", "smem", 2 * (256 + 1) * 4, 16, "kernel");
+PL_USES("pipelink_mok_fw_sched");
+PL_FACT("mok.framework.MAX_EXPERTS", 256);
+PL_PRELUDE("../include/mok_abi.h");
+PL_PRELUDE("../include/mok_device.hpp");
+PL_EMIT_MAIN()

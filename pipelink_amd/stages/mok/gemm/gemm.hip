@@ -17,6 +17,8 @@
 // makes a fragment read (32 consecutive rows, one chunk each) touch 16 different 16-byte
 // bank groups per 16 lanes.  The depth is a link-time handle; the ring offset inside the
 // workgroup's dynamic LDS is another.
+#include <pipelink/stage.hpp>
+#ifndef PIPELINK_EMIT
 #include "../include/mok_device.hpp"
 
 extern "C" __device__ int pipelink_mok_gemm_depth();  // ring slots (2 or 3), bound at link time
@@ -32,10 +34,16 @@ constexpr int X_GROUPS = TILE_X / 8 / WAVES;  // 8-row load groups per wave (4)
 constexpr int W_GROUPS = TILE_W / 8 / WAVES;  // (4)
 constexpr int LOADS_PER_SLOT = X_GROUPS + W_GROUPS + 1;  // + one dword of scales per lane
 
+// Addresses are a wave-uniform base (kept in scalar registers) plus a 32-bit lane offset: one
+// operand of one expert is far below 4 GiB, and 8 + 1 offsets cost half the vector registers
+// of 9 pointers.
 struct Loader {
-  const uint8_t* xsrc[X_GROUPS];  // this lane's 16 bytes of its row in each group, at k = 0
-  const uint8_t* wsrc[W_GROUPS];
-  const uint8_t* scsrc;           // scale row of this thread's row (threads 0..255 rows, 256..511 weights)
+  const uint8_t* xbase;           // activations (all rows)
+  const uint8_t* wbase;           // this expert's weight matrix (gate or up or down, by wave)
+  const uint8_t* scbase;          // scale matrix this thread's row belongs to
+  uint32_t xsrc[X_GROUPS];        // this lane's 16 bytes of its row in each group, at k = 0
+  uint32_t wsrc[W_GROUPS];
+  uint32_t scsrc;                 // scale row of this thread's row (threads 0..255 rows, 256..511 weights)
   int chunk_byte;                 // byte offset inside the 128-byte line this lane fetches in even groups
   int xdst, wdst, scdst;          // slot-relative LDS byte offsets of the wave's first group
 };
@@ -49,11 +57,11 @@ __device__ __forceinline__ void issue_slot(const Loader& ld, unsigned char* slot
   // the lane's chunk there is the even-group chunk with bit 2 (64 bytes) flipped
 #pragma unroll
   for (int j = 0; j < X_GROUPS; ++j)
-    if ((ld.chunk_byte ^ ((j & 1) << 6)) < k_left) load16_to_lds(ld.xsrc[j] + kbyte, slot + ld.xdst + j * 1024);
+    if ((ld.chunk_byte ^ ((j & 1) << 6)) < k_left) load16_to_lds(ld.xbase + kbyte + ld.xsrc[j], slot + ld.xdst + j * 1024);
 #pragma unroll
   for (int j = 0; j < W_GROUPS; ++j)
-    if ((ld.chunk_byte ^ ((j & 1) << 6)) < k_left) load16_to_lds(ld.wsrc[j] + kbyte, slot + ld.wdst + j * 1024);
-  load4_to_lds(ld.scsrc + (kbyte >> 5), slot + ld.scdst);
+    if ((ld.chunk_byte ^ ((j & 1) << 6)) < k_left) load16_to_lds(ld.wbase + kbyte + ld.wsrc[j], slot + ld.wdst + j * 1024);
+  load4_to_lds(ld.scbase + (kbyte >> 5) + ld.scsrc, slot + ld.scdst);
 }
 
 // MFMA 32x32x64 f8f6f4 operand of lane (row = lane % 32, half = lane / 32): registers 0-3
@@ -131,8 +139,9 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       int row = t.row_begin + trow;
       row = row < t.row_end ? row : t.row_end - 1;
       const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
-      ld.xsrc[j] = act.q + (int64_t)src * act.ld_q + 16 * (pos ^ swizzle(trow));
+      ld.xsrc[j] = (uint32_t)src * (uint32_t)act.ld_q + 16 * (pos ^ swizzle(trow));
     }
+    ld.xbase = act.q;
     ld.xdst = wave * X_GROUPS * 1024;
     const MokMxView& wv = gate_up ? (wave < WAVES / 2 ? g.w_gate : g.w_up) : g.w_down;
 #pragma unroll
@@ -140,21 +149,24 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       const int wl = (wave * W_GROUPS + j) * 8 + lrow;  // tile-local weight row
       int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
       col = col < wv.rows ? col : wv.rows - 1;
-      ld.wsrc[j] = wv.q + (int64_t)t.expert * wv.expert_pitch_q + (int64_t)col * wv.ld_q + 16 * (pos ^ swizzle(wl));
+      ld.wsrc[j] = (uint32_t)col * (uint32_t)wv.ld_q + 16 * (pos ^ swizzle(wl));
     }
+    ld.wbase = wv.q + (int64_t)t.expert * wv.expert_pitch_q;
     ld.wdst = SLOT_X_BYTES + wave * W_GROUPS * 1024;
     // scales: thread tid < 256 fetches routed row tid's dword, the others weight row tid - 256
     if (tid < TILE_X) {
       int row = t.row_begin + tid;
       row = row < t.row_end ? row : t.row_end - 1;
       const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
-      ld.scsrc = act.sc + (int64_t)src * act.ld_sc;
+      ld.scbase = act.sc;
+      ld.scsrc = (uint32_t)src * (uint32_t)act.ld_sc;
     } else {
       const int wl = tid - TILE_X;
       const MokMxView& sv = gate_up ? (wl < TILE_W / 2 ? g.w_gate : g.w_up) : g.w_down;
       int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
       col = col < sv.rows ? col : sv.rows - 1;
-      ld.scsrc = sv.sc + (int64_t)t.expert * sv.expert_pitch_sc + (int64_t)col * sv.ld_sc;
+      ld.scbase = sv.sc + (int64_t)t.expert * sv.expert_pitch_sc;
+      ld.scsrc = (uint32_t)col * (uint32_t)sv.ld_sc;
     }
     ld.scdst = SLOT_X_BYTES + SLOT_W_BYTES + wave * 256;
   }
@@ -258,3 +270,27 @@ extern "C" __device__ void mok_gemm_fwd(const void* view, const MokGemmTask* tas
     mok_gemm_owner::mainloop<3>(g, *task, *acc);  // needs 3 x 66 KB: beyond one CU's LDS at this tile size
   if (task->op == MOK_GEMM_FWD_ROUTED_DOWN) mok_gemm_owner::store_down(g, *task, *acc);
 }
+#else  // PIPELINK_EMIT: host-evaluated annotations only
+#include "../include/mok_abi.h"
+#endif
+
+PL_STAGE("mok.gemm", "0.1.0");
+PL_PARAMS(MokGemmResidue);
+PL_TOPOLOGY(true, "static");
+PL_VARIANT(0, {{"pipelink_mok_precision", 1}});  // MXFP8 (campaigns/mok/port/include/mok_abi.h: MOK_PRECISION_MXFP8)
+PL_EXPORT(mok_gemm_init, mok_gemm_init, "extern \"C\" __device__ void mok_gemm_init(const void* view);");
+PL_EXPORT(mok_gemm_fwd, mok_gemm_fwd,
+          "extern \"C\" __device__ void mok_gemm_fwd(const void* view, const MokGemmTask* task, "
+          "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc);");
+PL_SERVE(gemm_init, "mok_gemm_init");
+PL_SERVE(gemm_fwd, "mok_gemm_fwd");
+// ring of `depth` slots: 256 x 128 B of routed rows, 256 x 128 B of weight rows, 2 KB of scales
+PL_CLAIM_RING("pipelink_mok_gemm_arena", "smem", 0, "pipelink_mok_gemm_depth", 67584, 1024, "kernel");
+PL_USES("pipelink_mok_gemm_depth");
+PL_USES("pipelink_mok_gemm_arena");
+PL_FACT("mok.gemm.TILE_X", 256);
+PL_FACT("mok.gemm.TILE_W", 256);
+PL_FACT("mok.gemm.K_SLOT", 128);
+PL_PRELUDE("../include/mok_abi.h");
+PL_PRELUDE("../include/mok_device.hpp");
+PL_EMIT_MAIN()
