@@ -180,7 +180,7 @@ def _check_slots(handle: str, depth_ident, pipeline: Pipeline, claims: dict[str,
         _reject(path, "barrier slots extent must equal the ring depth", handle=handle)
 
 
-def expand(channel: Channel, pipeline: Pipeline, stages: list[Stage], seen_inits: dict[tuple, str] | None = None
+def expand(channel: Channel, pipeline: Pipeline, stages: list[Stage], seen_inits: dict[tuple, tuple] | None = None
            ) -> Expansion:
     """Expand one paired channel or raise ``SolveError`` with ``L-PROTO`` failures."""
     name = channel.name
@@ -241,11 +241,12 @@ def expand(channel: Channel, pipeline: Pipeline, stages: list[Stage], seen_inits
         if pi.get("owner") is None and pi.get("warp") is None:
             _reject(f"{path}.protocol.init", "init requires an owner or a physical initializing warp")
         if seen_inits is not None:
+            # several channels may ride one physical ring of slots, but it is initialised once
             key = (result["full"][0], result["empty"][0])
-            if key in seen_inits and seen_inits[key] != name:
-                _reject(f"{path}.protocol.init", "barrier ring has more than one init owner or materializer",
-                        other=seen_inits[key])
-            seen_inits[key] = name
+            if key in seen_inits and seen_inits[key][1] != pi:
+                _reject(f"channels.{seen_inits[key][0]}.protocol.init",
+                        "barrier ring has more than one init owner or materializer", expected=pi, actual=seen_inits[key][1])
+            seen_inits.setdefault(key, (name, pi))
         return Expansion(name, kind, tx_full=result["full"][2], tx_empty=result["empty"][2],
                          arrive_full=result["full"][1], arrive_empty=result["empty"][1], init_owner=pi.get("owner"),
                          init_materializer=pi["materializer"], slots=(result["full"][0], result["empty"][0]),
@@ -294,5 +295,5 @@ def expand(channel: Channel, pipeline: Pipeline, stages: list[Stage], seen_inits
 
 
 def expand_all(channels: dict[str, Channel], pipeline: Pipeline, stages: list[Stage]) -> list[Expansion]:
-    seen: dict[tuple, str] = {}
+    seen: dict[tuple, tuple] = {}
     return [expand(channels[name], pipeline, stages, seen) for name in sorted(channels)]

@@ -1,0 +1,141 @@
+"""Host-less launch of a linked pipeline: no provider libraries, the caller supplies buffers and
+a function that turns their device addresses into per-stage params blobs.
+
+Mirrors pipec/src/pipec2/launcher.py:107-333 of the reference: ``open_hostless`` allocates and
+uploads (arrays) or zeroes (shape/dtype specs) every buffer *before* ``params(addresses)`` runs,
+checks that the returned blobs cover exactly the non-empty entries of ``link.json``'s
+``params.entries`` (else ``L-PARAMS`` at ``launch.params``), copies them to their linked offsets
+and returns a ``HostlessSession`` with ``launch / synchronize / read / write / time / with_image /
+close``.  ``with_image`` loads a second code object that shares buffers, params and stream --
+the linked-versus-one-unit A/B switch.  The backend is anything with the ``HipBackend`` method
+set, so the CPU tests drive it with an in-memory fake."""
+from __future__ import annotations
+
+import json
+from pathlib import Path
+from typing import Any, Callable
+
+import numpy as np
+
+from .clauses import ClauseFailure, LaunchError
+
+
+def _fail(clause: str, path: str, message: str, **detail: Any):
+    raise LaunchError([ClauseFailure(clause, path, message, detail)])
+
+
+class HostlessSession:
+    def __init__(self, backend, link: dict[str, Any], function: int, module: int, buffers: dict[str, tuple[int, int, Any]],
+                 params_addr: int, grid: tuple[int, int, int], owns: bool = True):
+        self.backend, self.link, self._fn, self._module = backend, link, function, module
+        self.buffers, self.params_addr, self.grid, self._owns = buffers, params_addr, grid, owns
+        self._children: list[HostlessSession] = []
+
+    def launch(self) -> None:
+        self.backend.launch(self._fn, self.params_addr, self.grid, (self.link["threads"], 1, 1), self.link["dyn_smem_bytes"])
+
+    def synchronize(self) -> None:
+        self.backend.synchronize()
+
+    def read(self, name: str) -> np.ndarray:
+        addr, size, spec = self.buffers[name]
+        shape, dtype = spec
+        return np.frombuffer(self.backend.readback(addr, size), dtype=dtype).reshape(shape).copy()
+
+    def write(self, name: str, array: np.ndarray) -> None:
+        addr, size, spec = self.buffers[name]
+        data = np.ascontiguousarray(array, dtype=spec[1])
+        if data.nbytes != size:
+            _fail("L-LAUNCH", f"launch.buffers.{name}", "array size differs from the buffer's")
+        self.backend.upload(addr, data.tobytes())
+
+    def time(self, n: int) -> float:
+        """Milliseconds per launch over n back-to-back launches (one event pair)."""
+        if n <= 0:
+            _fail("L-LAUNCH", "launch.time", "launch count must be positive")
+        e0, e1 = self.backend.event_create(), self.backend.event_create()
+        self.backend.event_record(e0)
+        for _ in range(n):
+            self.launch()
+        self.backend.event_record(e1)
+        self.backend.event_synchronize(e1)
+        ms = self.backend.event_elapsed_time(e0, e1) / n
+        self.backend.event_destroy(e0)
+        self.backend.event_destroy(e1)
+        if not (ms > 0 and np.isfinite(ms)):
+            _fail("L-LAUNCH", "launch.time", "measured time is not finite and positive")
+        return ms
+
+    def with_image(self, image_path: str | Path) -> "HostlessSession":
+        module = self.backend.module_load(Path(image_path).read_bytes())
+        fn = self.backend.module_function(module, self.link["kernel_symbol"], self.link["dyn_smem_bytes"])
+        child = HostlessSession(self.backend, self.link, fn, module, self.buffers, self.params_addr, self.grid, owns=False)
+        self._children.append(child)
+        return child
+
+    def close(self) -> None:
+        for c in self._children:
+            c.close()
+        self._children.clear()
+        self.backend.module_unload(self._module)
+        if self._owns:
+            for addr, _, _ in self.buffers.values():
+                self.backend.free(addr)
+            self.backend.free(self.params_addr)
+
+
+def open_hostless(link_json: str | Path | dict, *, buffers: dict[str, Any], params: Callable[[dict[str, int]], dict[str, bytes]],
+                  grid: tuple[int, ...], backend=None, image: str | Path | None = None, device: int = 0) -> HostlessSession:
+    if isinstance(link_json, dict):
+        link, base = link_json, Path(".")
+    else:
+        link, base = json.loads(Path(link_json).read_text()), Path(link_json).parent
+    if link.get("host"):
+        _fail("L-LAUNCH", "launch.host", "link carries a host section: open it through its providers")
+    if backend is None:
+        from ..host.backend import HipBackend
+        backend = HipBackend(device)
+    backend.current()
+    placed: dict[str, tuple[int, int, Any]] = {}
+    for name, spec in buffers.items():
+        if isinstance(spec, np.ndarray):
+            data = np.ascontiguousarray(spec)
+            addr = backend.allocate(max(data.nbytes, 1))
+            backend.upload(addr, data.tobytes())
+            placed[name] = (addr, data.nbytes, (data.shape, data.dtype))
+        else:
+            shape, dtype = spec
+            size = int(np.prod(shape)) * np.dtype(dtype).itemsize
+            addr = backend.allocate(max(size, 1))
+            backend.zero(addr, size)
+            placed[name] = (addr, size, (tuple(shape), np.dtype(dtype)))
+    backend.synchronize()
+    blobs = params({n: a for n, (a, _, _) in placed.items()})
+    entries = {e["stage_id"]: e for e in link["params"]["entries"] if e["bytes"]}
+    if set(blobs) != set(entries):
+        _fail("L-PARAMS", "launch.params", "params blobs do not cover exactly the linked params entries",
+              expected=sorted(entries), actual=sorted(blobs))
+    image_bytes = bytearray(max(link["params"]["total_bytes"], 16))
+    for sid, blob in blobs.items():
+        e = entries[sid]
+        if len(blob) != e["bytes"]:
+            _fail("L-PARAMS", f"launch.params.{sid}", "params blob size differs from the packed layout",
+                  expected=e["bytes"], actual=len(blob))
+        image_bytes[e["offset"]:e["offset"] + e["bytes"]] = blob
+    params_addr = backend.allocate(len(image_bytes))
+    backend.upload(params_addr, bytes(image_bytes))
+    path = Path(image) if image else base / link["target"]["image"]
+    module = backend.module_load(path.read_bytes())
+    fn = backend.module_function(module, link["kernel_symbol"], link["dyn_smem_bytes"])
+    g = tuple(grid) + (1,) * (3 - len(grid))
+    return HostlessSession(backend, link, fn, module, placed, params_addr, g)
+
+
+def run_hostless(link_json, *, buffers, params, grid, outputs: list[str], **kw) -> dict[str, np.ndarray]:
+    s = open_hostless(link_json, buffers=buffers, params=params, grid=grid, **kw)
+    try:
+        s.launch()
+        s.synchronize()
+        return {n: s.read(n) for n in outputs}
+    finally:
+        s.close()
