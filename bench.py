@@ -36,7 +36,7 @@ def make_inputs(dev, seed=0):
     time); quantised on the device (bit-exact with the host rule) into 128-byte-pitched rows."""
     import torch
     from pipelink_amd.host import mok_inputs
-    from pipelink_amd.host.mok import code_pitch, mxfp8_quantize_device
+    from pipelink_amd.host.mok import code_pitch, mxfp8_quantize_device, weight_scales_to_slot_major
 
     g = torch.Generator().manual_seed(seed)
     logits = torch.randn(T, E, generator=g)
@@ -51,16 +51,18 @@ def make_inputs(dev, seed=0):
             q, sc = mxfp8_quantize_device(w.to(dev), code_pitch(k))
             qs.append(q)
             scs.append(sc)
-        return torch.stack(qs), torch.stack(scs)
+        return torch.stack(qs), torch.stack(scs), weight_scales_to_slot_major(torch.stack(scs), k)
 
     wg = weights(I, H)
     wu = weights(I, H)
     wd = weights(H, I)
-    return dict(tokens_per_expert=counts.to(dev), row_token=row_token.to(dev), x_q=x_q, x_sc=x_sc, w_gate_q=wg[0],
-                w_gate_sc=wg[1], w_up_q=wu[0], w_up_sc=wu[1], w_down_q=wd[0], w_down_sc=wd[1])
+    dev_args = dict(tokens_per_expert=counts.to(dev), row_token=row_token.to(dev), x_q=x_q, x_sc=x_sc, w_gate_q=wg[0],
+                    w_gate_sc=wg[2], w_up_q=wu[0], w_up_sc=wu[2], w_down_q=wd[0], w_down_sc=wd[2])
+    row_major = dict(w_gate_sc=wg[1], w_up_sc=wu[1], w_down_sc=wd[1])  # what the CPU oracle reads
+    return dev_args, row_major
 
 
-def cpu_baseline(inp, sample_tokens=1024, reps=3):
+def cpu_baseline(inp, row_major, sample_tokens=1024, reps=3):
     """The oracle on the host cores, first `sample_tokens` tokens of the same inputs."""
     import numpy as np
     import torch
@@ -72,7 +74,7 @@ def cpu_baseline(inp, sample_tokens=1024, reps=3):
     g = torch.Generator().manual_seed(0)
     logits = torch.randn(T, E, generator=g)[:sample_tokens]
     counts, row_token = mok_inputs.route(logits, TOPK)
-    host = {k: v.cpu() for k, v in inp.items()}
+    host = {k: v.cpu() for k, v in {**inp, **row_major}.items()}
     args = dict(x_q=host["x_q"][:sample_tokens, :H], x_sc=host["x_sc"][:sample_tokens],
                 wg_q=host["w_gate_q"][:, :, :H], wg_sc=host["w_gate_sc"], wu_q=host["w_up_q"][:, :, :H],
                 wu_sc=host["w_up_sc"], wd_q=host["w_down_q"][:, :, :I], wd_sc=host["w_down_sc"], counts=counts,
@@ -111,7 +113,7 @@ def main() -> int:
 
     paths = mok_build.images()  # raises if the HIP images are missing: there is no fallback path
     dev = torch.device("cuda:0")
-    inp = make_inputs(dev)
+    inp, row_major = make_inputs(dev)
     rows = T * TOPK
     hq = torch.zeros((rows, code_pitch(I)), dtype=torch.uint8, device=dev)
     hsc = torch.zeros((rows, scale_pitch(I)), dtype=torch.uint8, device=dev)
@@ -184,7 +186,7 @@ def main() -> int:
         "linked_over_one_unit": pair,
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(inp)
+        out["cpu_baseline"] = cpu_baseline(inp, row_major)
     print(json.dumps(out))
     linked.close()
     control.close()

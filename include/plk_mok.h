@@ -13,8 +13,11 @@
  * Operand layouts (all row-major; a code row may be padded to a pitch ld_q >= K, a multiple
  * of 16 -- a pitch that is a multiple of 128 makes every ring-slot row one aligned cache
  * line, which is what the loader is fastest on):
- *   x_q [T,H] e4m3, x_sc [T,ld_sc_h] e8m0 (one byte per 32 elements of H; ld_sc_h % 4 == 0)
- *   w_gate_q / w_up_q [E,I,H], scales [E,I,ld_sc_h];  w_down_q [E,H,I], scales [E,H,ld_sc_i]
+ *   x_q [T,H] e4m3, x_sc [T,ld_sc_h] e8m0 (one byte per 32 elements of H; ld_sc_h % 16 == 0)
+ *   w_gate_q / w_up_q [E,I,H], w_down_q [E,H,I]; weight scales are SLOT-MAJOR:
+ *   [E, ceil(K/128), N, 4] (the 4 scale bytes of one 128-element K-slot of one row are a dword,
+ *   and one slot's dwords of consecutive rows are contiguous) -- convert a row-major scale
+ *   matrix once, when the weights are loaded, with plk_mxfp8_scales_to_slot_major
  *   tokens_per_expert [E] i32, row_token [R] i32 (routed row -> token; 0 = rows are tokens)
  *   hidden_q [R,I] e4m3 + hidden_sc [R,ld_sc_i] (written by pass 1, read by pass 2)
  *   y [R,H] bf16 */
@@ -71,6 +74,11 @@ int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass,
  * (padding bytes zeroed). */
 int plk_mxfp8_quantize(uint64_t src, int src_is_bf16, int64_t rows, int32_t k, uint64_t dst_q, int32_t ld_q,
                        uint64_t dst_sc, int32_t ld_sc, void* stream);
+
+/* Row-major e8m0 scales src [rows, ld_sc] -> slot-major dst [ceil(k/128), rows, 4] (pad bytes 0).
+ * For a weight tensor [E, N, K] call it once per expert (or once with rows = E*N when the
+ * caller wants one slot-major block per expert, use rows = N and offset the pointers). */
+int plk_mxfp8_scales_to_slot_major(uint64_t src, int64_t rows, int32_t k, int32_t ld_sc, uint64_t dst, void* stream);
 
 #ifdef __cplusplus
 }

@@ -38,8 +38,8 @@ static int check_problem(const plk_mok_problem* p) {
     return plk_hip_set_error(PLK_E_CAPACITY, "plk_mok: num_experts must be in 1..256");
   if (p->hidden <= 0 || p->intermediate <= 0 || p->hidden % K_STEP || p->intermediate % K_STEP)
     return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: hidden and intermediate must be positive multiples of 64");
-  if (p->ld_sc_h % 4 || p->ld_sc_i % 4 || p->ld_sc_h * 32 < p->hidden || p->ld_sc_i * 32 < p->intermediate)
-    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: scale pitch must be a multiple of 4 covering K/32 blocks");
+  if (p->ld_sc_h % 16 || p->ld_sc_i % 16 || p->ld_sc_h * 32 < p->hidden || p->ld_sc_i * 32 < p->intermediate)
+    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: scale pitch must be a multiple of 16 covering K/32 blocks");
   if ((p->ld_q_h && (p->ld_q_h < p->hidden || p->ld_q_h % 16)) || (p->ld_q_i && (p->ld_q_i < p->intermediate || p->ld_q_i % 16)))
     return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: code row pitch must be a multiple of 16 and at least K");
   if (p->num_tokens < 0 || p->routed_rows < 0)
@@ -51,6 +51,7 @@ static int check_problem(const plk_mok_problem* p) {
   return PLK_OK;
 }
 
+// activations: row-major scales with pitch ld_sc; weights (per_expert): slot-major scales [slots, rows, 4]
 static MokMxView view(uint64_t q, uint64_t sc, int64_t rows, int k, int ld_q, int ld_sc, bool per_expert) {
   MokMxView v{};
   v.q = (const uint8_t*)(uintptr_t)q;
@@ -60,7 +61,7 @@ static MokMxView view(uint64_t q, uint64_t sc, int64_t rows, int k, int ld_q, in
   v.ld_q = ld_q;
   v.ld_sc = ld_sc;
   v.expert_pitch_q = per_expert ? rows * (int64_t)ld_q : 0;
-  v.expert_pitch_sc = per_expert ? rows * (int64_t)ld_sc : 0;
+  v.expert_pitch_sc = per_expert ? (int64_t)((k + 127) / 128) * rows * 4 : 0;
   return v;
 }
 
@@ -239,6 +240,37 @@ extern "C" int plk_mxfp8_quantize(uint64_t src, int src_is_bf16, int64_t rows, i
   else
     mxfp8_quantize_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>(
         (const void*)(uintptr_t)src, rows, k, (uint8_t*)(uintptr_t)dst_q, ld_q, (uint8_t*)(uintptr_t)dst_sc, ld_sc);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return plk_hip_set_error(PLK_E_RESOURCE, hipGetErrorString(e));
+  return PLK_OK;
+}
+
+// ---- scale layout conversion ---------------------------------------------------------------
+__global__ void __launch_bounds__(256) scales_to_slot_major_kernel(const uint8_t* __restrict__ src, int64_t rows, int nblocks,
+                                                                    int ld_sc, uint32_t* __restrict__ dst, int nslots) {
+  const int64_t total = rows * (int64_t)nslots;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t s = i / rows, r = i - s * rows;
+    uint32_t v = 0;
+    for (int j = 0; j < 4; ++j) {
+      const int b = (int)s * 4 + j;
+      if (b < nblocks) v |= (uint32_t)src[r * ld_sc + b] << (8 * j);
+    }
+    dst[i] = v;
+  }
+}
+
+extern "C" int plk_mxfp8_scales_to_slot_major(uint64_t src, int64_t rows, int32_t k, int32_t ld_sc, uint64_t dst,
+                                              void* stream) {
+  if (rows < 0 || k <= 0 || k % 32 || ld_sc * 32 < k)
+    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mxfp8_scales_to_slot_major: k must be a positive multiple of 32 covered by ld_sc");
+  if (rows == 0) return PLK_OK;
+  if (!src || !dst) return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mxfp8_scales_to_slot_major: null device address");
+  const int nslots = (k + 127) / 128;
+  int64_t grid = (rows * nslots + 255) / 256;
+  if (grid > 65536) grid = 65536;
+  scales_to_slot_major_kernel<<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>(
+      (const uint8_t*)(uintptr_t)src, rows, k / 32, ld_sc, (uint32_t*)(uintptr_t)dst, nslots);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return plk_hip_set_error(PLK_E_RESOURCE, hipGetErrorString(e));
   return PLK_OK;

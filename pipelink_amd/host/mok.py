@@ -19,8 +19,26 @@ MX_BLOCK = 32
 
 
 def scale_pitch(k: int) -> int:
-    """Bytes per scale row: K/32 rounded up to a multiple of 4."""
-    return ((k // MX_BLOCK) + 3) // 4 * 4
+    """Bytes per row-major scale row: K/32 rounded up to a multiple of 16."""
+    return ((k // MX_BLOCK) + 15) // 16 * 16
+
+
+def scale_slots(k: int) -> int:
+    """Number of 128-element ring slots along K (= dwords per row of a slot-major scale array)."""
+    return (k + 127) // 128
+
+
+def weight_scales_to_slot_major(sc: torch.Tensor, k: int) -> torch.Tensor:
+    """Row-major weight scales [E, N, ld] -> the slot-major layout the GEMM reads, [E, K/128, N, 4]."""
+    if not sc.is_cuda or not sc.is_contiguous() or sc.dim() != 3 or sc.dtype != torch.uint8:
+        raise PlkError(3, "scales must be a contiguous 3-D uint8 device tensor")
+    e, n, ld = sc.shape
+    out = torch.empty((e, scale_slots(k), n, 4), dtype=torch.uint8, device=sc.device)
+    lib = load_library()
+    stream = c_void_p(torch.cuda.current_stream().cuda_stream)
+    for i in range(e):
+        check(lib, lib.plk_mxfp8_scales_to_slot_major(sc[i].data_ptr(), n, k, ld, out[i].data_ptr(), stream))
+    return out
 
 
 def link_info_from_json(link: dict) -> MokLinkInfo:
@@ -76,9 +94,11 @@ class MoKSession:
         if hidden_q.shape[0] != r or y.dtype != torch.bfloat16 or ldh < h or ldi_q < i:
             raise PlkError(3, "hidden_q / y shapes disagree")
         ldsh, ldsi = scale_pitch(h), scale_pitch(i)
-        if x_sc.shape[1] != ldsh or w_gate_sc.shape[2] != ldsh or w_up_sc.shape[2] != ldsh or \
-                w_down_sc.shape[2] != ldsi or hidden_sc.shape[1] != ldsi:
-            raise PlkError(3, "scale pitch must be K/32 rounded up to a multiple of 4")
+        if x_sc.shape[1] != ldsh or hidden_sc.shape[1] != ldsi:
+            raise PlkError(3, "activation scale pitch must be K/32 rounded up to a multiple of 16")
+        if tuple(w_gate_sc.shape) != (e, scale_slots(h), i, 4) or tuple(w_up_sc.shape) != (e, scale_slots(h), i, 4) or \
+                tuple(w_down_sc.shape) != (e, scale_slots(i), h, 4):
+            raise PlkError(3, "weight scales must be slot-major [E, K/128, N, 4] (see weight_scales_to_slot_major)")
         if tokens_per_expert.dtype != torch.int32 or (row_token is not None and row_token.dtype != torch.int32):
             raise PlkError(3, "tokens_per_expert and row_token must be int32")
         return MokProblem(struct_bytes=sizeof(MokProblem), num_tokens=t_rows, hidden=h, intermediate=i, num_experts=e,

@@ -13,7 +13,7 @@ MX_BLOCK = 32
 
 
 def scale_pitch(k: int) -> int:
-    return ((k // MX_BLOCK) + 3) // 4 * 4
+    return ((k // MX_BLOCK) + 15) // 16 * 16
 
 
 def quantize(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:

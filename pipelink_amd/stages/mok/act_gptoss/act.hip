@@ -14,23 +14,39 @@
 #ifndef PIPELINK_EMIT
 #include "../include/mok_device.hpp"
 
-extern "C" __device__ int pipelink_mok_clamp();  // link-time variant: 1 = clamp to +-limit
+extern "C" __device__ int pipelink_mok_clamp();      // link-time variant: 1 = clamp to +-limit
+extern "C" __device__ int pipelink_mok_act_arena();  // byte offset of the staging tile in dynamic LDS
+
+extern __shared__ __attribute__((aligned(1024))) unsigned char pipelink_smem[];
 
 namespace mok_act_owner {
 using namespace mok;
 
 constexpr float SWIGLU_ALPHA = 1.702f;  // campaigns/mok/port/act_gptoss/swiglu.cuh:2
+constexpr int STAGE_PITCH = TILE_W / 2 + 16;            // bytes per staged row: 128 codes + pad against bank conflicts
+constexpr int STAGE_SCALE_OFF = TILE_X * STAGE_PITCH;   // [row][4] scale bytes behind the codes
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 template <bool CLAMPED>
 __device__ __forceinline__ float swiglu(float gate, float up, float limit) {
   if (CLAMPED) {
     gate = fminf(gate, limit);
-    up = fminf(fmaxf(up, -limit), limit);
+    up = __builtin_amdgcn_fmed3f(up, -limit, limit);
   }
-  // (up + 1) * gate * sigmoid(alpha * gate), fast exp and reciprocal as in the reference's
-  // --use_fast_math build (campaigns/mok/port/build.py:26)
-  const float den = 1.0f + __expf(-SWIGLU_ALPHA * gate);
+  // (up + 1) * gate * sigmoid(alpha * gate) with the hardware exp2 and reciprocal, as in the
+  // reference's --use_fast_math build (campaigns/mok/port/build.py:26)
+  const float den = 1.0f + __builtin_amdgcn_exp2f(gate * (-SWIGLU_ALPHA * 1.4426950408889634f));
   return (up + 1.0f) * (gate * __builtin_amdgcn_rcpf(den));
+}
+
+// round two floats to bf16 (nearest even, v_cvt_pk_bf16_f32) and widen them back
+__device__ __forceinline__ void bf16_round2(float& a, float& b) {
+  const f32x2 v = {a, b};
+  const uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  a = __uint_as_float(bits << 16);
+  b = __uint_as_float(bits & 0xFFFF0000u);
 }
 
 // e4m3 (OCP) pack of four floats already scaled into [-448, 448]
@@ -43,41 +59,69 @@ __device__ __forceinline__ uint32_t pack_e4m3x4(float a, float b, float c, float
 
 template <bool CLAMPED>
 __device__ __forceinline__ void forward(const MokActResidue& p, const MokActTask& t, const AccFrag& acc) {
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
   const int half = lane >> 5;
+  unsigned char* stage = pipelink_smem + pipelink_mok_act_arena();
+  // ---- activation + requant into an LDS tile [256 rows][128 codes] + [256 rows][4 scales] ----
 #pragma unroll
   for (int a = 0; a < 2; ++a) {  // gate fragments a, up fragments a + 2: same rows, same columns
-    const int col0 = t.col_begin + wrow0(wave, a);  // 32-column block of d_ff
+    const int tcol = wrow0(wave, a);  // tile-local first column of this 32-column block
 #pragma unroll
     for (int b = 0; b < XFRAGS; ++b) {
-      const int row = t.row_begin + xrow0(wave, b) + (lane & 31);
+      const int trow = xrow0(wave, b) + (lane & 31);
       float h[16];
       float amax = 0.0f;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        h[r] = bf16_round(swiglu<CLAMPED>(acc.v[a][b][r], acc.v[a + 2][b][r], p.swiglu_limit));
-        amax = fmaxf(amax, fabsf(h[r]));
+      for (int r = 0; r < 16; r += 2) {
+        h[r] = swiglu<CLAMPED>(acc.v[a][b][r], acc.v[a + 2][b][r], p.swiglu_limit);
+        h[r + 1] = swiglu<CLAMPED>(acc.v[a][b][r + 1], acc.v[a + 2][b][r + 1], p.swiglu_limit);
+        bf16_round2(h[r], h[r + 1]);  // the reference rounds to bf16 before quantising (swiglu.cuh:175)
+        amax = fmaxf(amax, fmaxf(fabsf(h[r]), fabsf(h[r + 1])));
       }
       // the other 16 columns of this row's block live in lane ^ 32
       amax = fmaxf(amax, __shfl_xor(amax, 32));
       int e = (int)((__float_as_uint(amax) >> 23) & 0xFFu) - 8;  // floor(log2(amax)) - 8 + 127
       e = e < 0 ? 0 : e;                                          // amax < 2^-118: scale byte 0
       const float inv = __uint_as_float((uint32_t)(254 - e) << 23);  // 2^(127 - e), e <= 247
-      const bool live = row < t.row_end && col0 < p.cols;
-      if (live) {
-        uint8_t* qrow = p.hidden_q + (int64_t)row * p.ld_q + col0 + 4 * half;
+      unsigned char* dst = stage + trow * STAGE_PITCH + tcol + 4 * half;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          float s[4];
+      for (int q = 0; q < 4; ++q) {
+        float s[4];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) s[j] = fminf(fmaxf(h[4 * q + j] * inv, -448.0f), 448.0f);
-          *reinterpret_cast<uint32_t*>(qrow + 8 * q) = pack_e4m3x4(s[0], s[1], s[2], s[3]);
-        }
-        if (half == 0) p.hidden_sc[(int64_t)row * p.ld_sc + (col0 >> 5)] = (uint8_t)e;
+        for (int j = 0; j < 4; ++j) s[j] = __builtin_amdgcn_fmed3f(h[4 * q + j] * inv, -448.0f, 448.0f);
+        *reinterpret_cast<uint32_t*>(dst + 8 * q) = pack_e4m3x4(s[0], s[1], s[2], s[3]);
+      }
+      if (half == 0) stage[STAGE_SCALE_OFF + trow * 4 + (tcol >> 5)] = (uint8_t)e;
+    }
+  }
+  __syncthreads();
+  // ---- coalesced write-out: a row is 128 bytes = 8 lanes x 16 bytes, 8 rows per wave store ----
+  const int chunk = lane & 7;
+  const bool col_ok = t.col_begin + chunk * 16 < p.cols;  // column extents are multiples of 32
+#pragma unroll
+  for (int it = 0; it < TILE_X / 64; ++it) {
+    const int trow = wave * (TILE_X / 8) + it * 8 + (lane >> 3);
+    const int row = t.row_begin + trow;
+    if (row < t.row_end && col_ok) {
+      const uint4 v = *reinterpret_cast<const uint4*>(stage + trow * STAGE_PITCH + chunk * 16);
+      *reinterpret_cast<uint4*>(p.hidden_q + (int64_t)row * p.ld_q + t.col_begin + chunk * 16) = v;
+    }
+  }
+  if (tid < TILE_X) {
+    const int row = t.row_begin + tid;
+    if (row < t.row_end) {
+      const uint32_t sc = *reinterpret_cast<const uint32_t*>(stage + STAGE_SCALE_OFF + tid * 4);
+      uint8_t* out = p.hidden_sc + (int64_t)row * p.ld_sc + (t.col_begin >> 5);
+      if (t.col_begin + TILE_W / 2 <= p.cols) {
+        *reinterpret_cast<uint32_t*>(out) = sc;  // col_begin is a multiple of 128: dword aligned
+      } else {
+        for (int j = 0; t.col_begin + 32 * j < p.cols; ++j) out[j] = (uint8_t)(sc >> (8 * j));
       }
     }
   }
+  __syncthreads();  // the staging tile shares LDS with the GEMM ring of the next tile
 }
 
 }  // namespace mok_act_owner
@@ -110,7 +154,10 @@ PL_EXPORT(mok_act_fwd, mok_act_fwd,
           "const MokCounters* counters, uint32_t* phase, const mok::AccFrag* acc);");
 PL_SERVE(act_init, "mok_act_init");
 PL_SERVE(act_fwd, "mok_act_fwd");
+// staging tile for the coalesced write-out; lives while no GEMM ring slot is in use
+PL_CLAIM("pipelink_mok_act_arena", "smem", 256 * 144 + 256 * 4, 1024, "phase:instr_act");
 PL_USES("pipelink_mok_clamp");
+PL_USES("pipelink_mok_act_arena");
 PL_PRELUDE("../include/mok_abi.h");
 PL_PRELUDE("../include/mok_device.hpp");
 PL_EMIT_MAIN()

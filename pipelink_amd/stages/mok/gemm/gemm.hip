@@ -9,9 +9,12 @@
 // four consecutive output columns of one routed row, which is what the requantising
 // epilogue and the bf16 store want.
 //
-// Ring: `depth` LDS slots of 66 KB.  A slot holds 128 contraction bytes of 256 routed rows
+// Ring: `depth` LDS slots of 65 KB.  A slot holds 128 contraction bytes of 256 routed rows
 // and of 256 weight rows, row-major (one 128-byte cache line per row), followed by one
-// dword of block scales (4 x e8m0) per row.  One global_load_lds_dwordx4 moves 8 rows:
+// dword of block scales (4 x e8m0) per weight row (weight scales are stored slot-major, so a
+// tile's 1 KB of them is one contiguous load).  The routed rows' scales are row-major in HBM
+// (rows are gathered); every fourth slot 16 bytes per row -- four slots' worth -- go to a
+// small double buffer behind the ring.  One global_load_lds_dwordx4 moves 8 rows:
 // eight lanes cover the 128 contiguous bytes of a row, so every L2 request is a full line.
 // The eight 16-byte chunks of a row are stored at position chunk ^ ((row / 2) % 8), which
 // makes a fragment read (32 consecutive rows, one chunk each) touch 16 different 16-byte
@@ -32,7 +35,7 @@ using namespace mok;
 constexpr int WAVES = THREADS / 64;
 constexpr int X_GROUPS = TILE_X / 8 / WAVES;  // 8-row load groups per wave (4)
 constexpr int W_GROUPS = TILE_W / 8 / WAVES;  // (4)
-constexpr int LOADS_PER_SLOT = X_GROUPS + W_GROUPS + 1;  // + one dword of scales per lane
+constexpr int LOADS_PER_SLOT = X_GROUPS + W_GROUPS + 2;  // upper bound: + weight scales + routed-row scales
 
 // Addresses are a wave-uniform base (kept in scalar registers) plus a 32-bit lane offset: one
 // operand of one expert is far below 4 GiB, and 8 + 1 offsets cost half the vector registers
@@ -40,19 +43,22 @@ constexpr int LOADS_PER_SLOT = X_GROUPS + W_GROUPS + 1;  // + one dword of scale
 struct Loader {
   const uint8_t* xbase;           // activations (all rows)
   const uint8_t* wbase;           // this expert's weight matrix (gate or up or down, by wave)
-  const uint8_t* scbase;          // scale matrix this thread's row belongs to
+  const uint8_t* xscbase;         // routed rows' scales, row-major
+  const uint8_t* wscbase;         // this lane's 16 bytes (4 rows) of the tile's weight scales in slot 0
+  uint32_t wsc_slot_pitch;        // bytes between two slots of the weight scales
+  uint32_t xscsrc;                // this thread's routed row in the scale matrix (threads 0..255)
   uint32_t xsrc[X_GROUPS];        // this lane's 16 bytes of its row in each group, at k = 0
   uint32_t wsrc[W_GROUPS];
-  uint32_t scsrc;                 // scale row of this thread's row (threads 0..255 rows, 256..511 weights)
   int chunk_byte;                 // byte offset inside the 128-byte line this lane fetches in even groups
-  int xdst, wdst, scdst;          // slot-relative LDS byte offsets of the wave's first group
+  int xdst, wdst;                 // slot-relative LDS byte offsets of the wave's first group
 };
 
 __device__ __forceinline__ int swizzle(int row) { return (row >> 1) & 7; }
 
 // Issue one slot.  k_left = contraction bytes from this slot's start to the end of the row:
 // the last slot of a K that is not a multiple of 128 only fetches the chunks that exist.
-__device__ __forceinline__ void issue_slot(const Loader& ld, unsigned char* slot, int kbyte, int k_left) {
+__device__ __forceinline__ void issue_slot(const Loader& ld, unsigned char* slot, unsigned char* xscale, int kbyte,
+                                           int k_left) {
   // group j starts at tile row 8 * (4 * wave + j): odd groups flip bit 2 of the swizzle, so
   // the lane's chunk there is the even-group chunk with bit 2 (64 bytes) flipped
 #pragma unroll
@@ -61,7 +67,12 @@ __device__ __forceinline__ void issue_slot(const Loader& ld, unsigned char* slot
 #pragma unroll
   for (int j = 0; j < W_GROUPS; ++j)
     if ((ld.chunk_byte ^ ((j & 1) << 6)) < k_left) load16_to_lds(ld.wbase + kbyte + ld.wsrc[j], slot + ld.wdst + j * 1024);
-  load4_to_lds(ld.scbase + (kbyte >> 5) + ld.scsrc, slot + ld.scdst);
+  const int wave = threadIdx.x >> 6;
+  const int s = kbyte >> 7;  // slot index
+  // wave 4: the tile's weight scales of this slot, 4 rows per lane
+  if (wave == 4) load16_to_lds(ld.wscbase + (size_t)s * ld.wsc_slot_pitch, slot + SLOT_X_BYTES + SLOT_W_BYTES);
+  // waves 0-3, every fourth slot: 16 scale bytes of each routed row (this slot and the next three)
+  if (wave < 4 && (s & 3) == 0) load16_to_lds(ld.xscbase + (kbyte >> 5) + ld.xscsrc, xscale + ((s >> 2) & 1) * (TILE_X * 16) + wave * 1024);
 }
 
 // MFMA 32x32x64 f8f6f4 operand of lane (row = lane % 32, half = lane / 32): registers 0-3
@@ -123,6 +134,7 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   const int K = act.k;
   const int nslots = (K + K_SLOT - 1) / K_SLOT;
   unsigned char* ring = pipelink_smem + pipelink_mok_gemm_arena();
+  unsigned char* xscale = ring + DEPTH * SLOT_BYTES;  // routed-row scale double buffer behind the ring
 
   // ---- loader addresses (fixed for the tile) ---------------------------------------
   // lane -> (row lane/8 of an 8-row group, LDS position lane%8); it fetches the chunk that
@@ -153,22 +165,23 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
     }
     ld.wbase = wv.q + (int64_t)t.expert * wv.expert_pitch_q;
     ld.wdst = SLOT_X_BYTES + wave * W_GROUPS * 1024;
-    // scales: thread tid < 256 fetches routed row tid's dword, the others weight row tid - 256
-    if (tid < TILE_X) {
-      int row = t.row_begin + tid;
+    // routed-row scales: thread tid < 256 fetches row tid's 16-byte piece
+    {
+      int row = t.row_begin + (tid & (TILE_X - 1));
       row = row < t.row_end ? row : t.row_end - 1;
       const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
-      ld.scbase = act.sc;
-      ld.scsrc = (uint32_t)src * (uint32_t)act.ld_sc;
-    } else {
-      const int wl = tid - TILE_X;
+      ld.xscbase = act.sc;
+      ld.xscsrc = (uint32_t)src * (uint32_t)act.ld_sc;
+    }
+    // weight scales, slot-major [slot][row][4]: lane l of one wave fetches tile rows 4l .. 4l+3
+    {
+      const int wl = 4 * lane;
       const MokMxView& sv = gate_up ? (wl < TILE_W / 2 ? g.w_gate : g.w_up) : g.w_down;
       int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
-      col = col < sv.rows ? col : sv.rows - 1;
-      ld.scbase = sv.sc + (int64_t)t.expert * sv.expert_pitch_sc;
-      ld.scsrc = (uint32_t)col * (uint32_t)sv.ld_sc;
+      col = col <= sv.rows - 4 ? col : sv.rows - 4;  // row counts are multiples of 32
+      ld.wscbase = sv.sc + (int64_t)t.expert * sv.expert_pitch_sc + (int64_t)col * 4;
+      ld.wsc_slot_pitch = (uint32_t)sv.rows * 4u;
     }
-    ld.scdst = SLOT_X_BYTES + SLOT_W_BYTES + wave * 256;
   }
 
   // ---- per-fragment LDS read offsets (step 0, first block) ---------------------------
@@ -177,13 +190,13 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   for (int b = 0; b < XFRAGS; ++b) {
     const int row = xrow0(wave, b) + r32;
     xoff[b] = row * K_SLOT + 16 * (half ^ swizzle(row));
-    xscoff[b] = SLOT_X_BYTES + SLOT_W_BYTES + row * 4;
+    xscoff[b] = row * 16;
   }
 #pragma unroll
   for (int a = 0; a < WFRAGS; ++a) {
     const int wl = wrow0(wave, a) + r32;
     woff[a] = SLOT_X_BYTES + wl * K_SLOT + 16 * (half ^ swizzle(wl));
-    wscoff[a] = SLOT_X_BYTES + SLOT_W_BYTES + TILE_X * 4 + wl * 4;
+    wscoff[a] = SLOT_X_BYTES + SLOT_W_BYTES + wl * 4;
   }
 
 #pragma unroll
@@ -196,7 +209,7 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   // ---- prologue: fill depth-1 slots ---------------------------------------------------
 #pragma unroll
   for (int s = 0; s < DEPTH - 1; ++s)
-    if (s < nslots) issue_slot(ld, ring + s * SLOT_BYTES, s * K_SLOT, K - s * K_SLOT);
+    if (s < nslots) issue_slot(ld, ring + s * SLOT_BYTES, xscale, s * K_SLOT, K - s * K_SLOT);
 
   int cur = 0;           // slot the next iteration consumes
   int fill = DEPTH - 1;  // slot the next issued load fills
@@ -208,7 +221,7 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       wait_vmcnt<0>();
     wg_barrier();  // slot i has landed for every wave; everyone is done reading slot i-1
     if (i + DEPTH - 1 < nslots)
-      issue_slot(ld, ring + fill * SLOT_BYTES, (i + DEPTH - 1) * K_SLOT, K - (i + DEPTH - 1) * K_SLOT);
+      issue_slot(ld, ring + fill * SLOT_BYTES, xscale, (i + DEPTH - 1) * K_SLOT, K - (i + DEPTH - 1) * K_SLOT);
     fill = fill + 1 == DEPTH ? 0 : fill + 1;
     const unsigned char* slot = ring + cur * SLOT_BYTES;
     cur = cur + 1 == DEPTH ? 0 : cur + 1;
@@ -217,7 +230,8 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
     // into bytes 0 and 2 where the MFMA's op_sel picks them
     int sx[XFRAGS], sw[WFRAGS];
 #pragma unroll
-    for (int b = 0; b < XFRAGS; ++b) sx[b] = (int)(*reinterpret_cast<const uint32_t*>(slot + xscoff[b]) >> (8 * half));
+    for (int b = 0; b < XFRAGS; ++b)
+      sx[b] = (int)(*reinterpret_cast<const uint32_t*>(xscale + ((i >> 2) & 1) * (TILE_X * 16) + xscoff[b] + 4 * (i & 3)) >> (8 * half));
 #pragma unroll
     for (int a = 0; a < WFRAGS; ++a) sw[a] = (int)(*reinterpret_cast<const uint32_t*>(slot + wscoff[a]) >> (8 * half));
     mma_step<false>(slot, xoff, woff, sx, sw, acc);
@@ -226,31 +240,51 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   wg_barrier();  // ring free for the next tile
 }
 
+// bf16 epilogue of the down op.  The accumulator is transposed through the (now idle) ring so
+// that the global stores are 16 bytes per lane and 512 contiguous bytes per routed row.
+constexpr int Y_PITCH = TILE_W * 2 + 16;  // bytes per staged row: 256 bf16 + pad against bank conflicts
+static_assert(TILE_X * Y_PITCH <= 2 * SLOT_BYTES + XSCALE_BYTES, "staging tile must fit the two-slot ring");
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  const f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // v_cvt_pk_bf16_f32, nearest even
+}
+
 __device__ __forceinline__ void store_down(const MokGemmResidue& g, const MokGemmTask& t, const AccFrag& acc) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
+  unsigned char* stage = pipelink_smem + pipelink_mok_gemm_arena();
 #pragma unroll
   for (int b = 0; b < XFRAGS; ++b) {
-    const int row = t.row_begin + xrow0(wave, b) + (lane & 31);
-    if (row >= t.row_end) continue;
-    uint16_t* yrow = g.y + (int64_t)row * g.ld_y;
+    unsigned char* rowp = stage + (xrow0(wave, b) + (lane & 31)) * Y_PITCH;
 #pragma unroll
     for (int a = 0; a < WFRAGS; ++a) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int col = t.col_begin + wrow0(wave, a) + 8 * q + 4 * (lane >> 5);
-        if (col >= g.w_down.rows) continue;  // columns come in groups of 4; extents are multiples of 32
-        uint32_t p0 = __float_as_uint(bf16_round(acc.v[a][b][4 * q + 0])) >> 16;
-        uint32_t p1 = __float_as_uint(bf16_round(acc.v[a][b][4 * q + 1])) & 0xFFFF0000u;
-        uint32_t p2 = __float_as_uint(bf16_round(acc.v[a][b][4 * q + 2])) >> 16;
-        uint32_t p3 = __float_as_uint(bf16_round(acc.v[a][b][4 * q + 3])) & 0xFFFF0000u;
+        const int col = wrow0(wave, a) + 8 * q + 4 * (lane >> 5);
         uint2 pk;
-        pk.x = p0 | p1;
-        pk.y = p2 | p3;
-        *reinterpret_cast<uint2*>(yrow + col) = pk;
+        pk.x = pack_bf16x2(acc.v[a][b][4 * q + 0], acc.v[a][b][4 * q + 1]);
+        pk.y = pack_bf16x2(acc.v[a][b][4 * q + 2], acc.v[a][b][4 * q + 3]);
+        *reinterpret_cast<uint2*>(rowp + col * 2) = pk;
       }
     }
   }
+  __syncthreads();
+  const int chunk = lane & 31;                              // 8 columns = 16 bytes
+  const bool col_ok = t.col_begin + chunk * 8 < g.w_down.rows;  // column extents are multiples of 32
+#pragma unroll 4
+  for (int it = 0; it < TILE_X / 16; ++it) {
+    const int trow = wave * (TILE_X / 8) + it * 2 + (lane >> 5);
+    const int row = t.row_begin + trow;
+    if (row < t.row_end && col_ok) {
+      const uint4 v = *reinterpret_cast<const uint4*>(stage + trow * Y_PITCH + chunk * 16);
+      *reinterpret_cast<uint4*>(g.y + (int64_t)row * g.ld_y + t.col_begin + chunk * 8) = v;
+    }
+  }
+  __syncthreads();  // the ring is reused by the next tile's loads
 }
 
 }  // namespace mok_gemm_owner
@@ -284,8 +318,9 @@ PL_EXPORT(mok_gemm_fwd, mok_gemm_fwd,
           "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc);");
 PL_SERVE(gemm_init, "mok_gemm_init");
 PL_SERVE(gemm_fwd, "mok_gemm_fwd");
-// ring of `depth` slots: 256 x 128 B of routed rows, 256 x 128 B of weight rows, 2 KB of scales
-PL_CLAIM_RING("pipelink_mok_gemm_arena", "smem", 0, "pipelink_mok_gemm_depth", 67584, 1024, "kernel");
+// ring of `depth` slots: 256 x 128 B of routed rows, 256 x 128 B of weight rows, 1 KB of weight scales
+// + 8 KB behind the ring: double buffer of the routed rows' scales
+PL_CLAIM_RING("pipelink_mok_gemm_arena", "smem", 8192, "pipelink_mok_gemm_depth", 66560, 1024, "phase:instr_gemm");
 PL_USES("pipelink_mok_gemm_depth");
 PL_USES("pipelink_mok_gemm_arena");
 PL_FACT("mok.gemm.TILE_X", 256);

@@ -50,9 +50,12 @@ typedef struct MokActTask {
 } MokActTask;
 #endif
 
-/* One MXFP8 operand: e4m3 codes [rows, k] (row pitch ld_q bytes) and e8m0 scales
- * [rows, ld_sc] (one byte per 32 k-elements, ld_sc a multiple of 4).  Weights carry an
- * expert pitch on both. */
+/* One MXFP8 operand: e4m3 codes [rows, k] (row pitch ld_q bytes) and e8m0 scales, one byte
+ * per 32 k-elements.  Activations keep their scales row-major [rows, ld_sc] with ld_sc a
+ * multiple of 16 (one 16-byte piece = the scales of four 128-element ring slots).  Weights
+ * keep them slot-major, [ceil(k/128), rows, 4] per expert, so the scales one workgroup tile
+ * needs for one ring slot are contiguous; ld_sc is unused for them.  Weights carry an expert
+ * pitch on both arrays. */
 typedef struct MokMxView {
   const uint8_t* q;
   const uint8_t* sc;

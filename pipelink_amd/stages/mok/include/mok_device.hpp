@@ -27,8 +27,9 @@ constexpr int XFRAGS = 2;       // 32-row activation fragments per wave
 constexpr int THREADS = 512;
 constexpr int SLOT_X_BYTES = TILE_X * K_SLOT;
 constexpr int SLOT_W_BYTES = TILE_W * K_SLOT;
-constexpr int SLOT_SCALE_BYTES = (TILE_X + TILE_W) * 4;  // one dword (4 block scales) per row
-constexpr int SLOT_BYTES = SLOT_X_BYTES + SLOT_W_BYTES + SLOT_SCALE_BYTES;  // 67584
+constexpr int SLOT_SCALE_BYTES = TILE_W * 4;             // one dword (4 block scales) per weight row
+constexpr int SLOT_BYTES = SLOT_X_BYTES + SLOT_W_BYTES + SLOT_SCALE_BYTES;  // 66560
+constexpr int XSCALE_BYTES = 2 * TILE_X * 16;            // two buffers of 16 scale bytes (4 slots) per routed row
 
 // fp32 accumulator of one wave: [weight fragment][row fragment] MFMA 32x32 C tiles.
 // Element (reg r, lane l) of tile (a, b) is

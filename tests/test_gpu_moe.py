@@ -31,10 +31,13 @@ def cell():
 
 
 def _run(sess, inp, H, I, pitch_h=None, pitch_i=None, limit=7.0):
-    from pipelink_amd.host.mok import scale_pitch
+    from pipelink_amd.host.mok import scale_pitch, weight_scales_to_slot_major
 
     dev = torch.device("cuda:0")
     d = {k: v.to(dev) for k, v in inp.__dict__.items()}
+    d["w_gate_sc"] = weight_scales_to_slot_major(d["w_gate_sc"], H)   # the layout the GEMM reads
+    d["w_up_sc"] = weight_scales_to_slot_major(d["w_up_sc"], H)
+    d["w_down_sc"] = weight_scales_to_slot_major(d["w_down_sc"], I)
     if pitch_h:  # re-pitch the K = H operands
         def pad(t, p):
             out = torch.zeros(t.shape[:-1] + (p,), dtype=torch.uint8, device=dev)
@@ -127,7 +130,8 @@ def test_device_quantiser_is_bit_exact():
     for src in (x, x.to(torch.bfloat16)):
         q, sc = mxfp8_quantize_device(src.cuda())
         oq, osc = mxfp8.mx_quantize(src.float().numpy())
-        assert np.array_equal(q.cpu().numpy(), oq) and np.array_equal(sc.cpu().numpy(), osc)
+        assert np.array_equal(q.cpu().numpy(), oq) and np.array_equal(sc.cpu().numpy()[:, :90], osc[:, :90])
+        assert not sc.cpu().numpy()[:, 90:].any()   # pad bytes of the 16-byte-pitched scale rows are zero
     q, sc = mxfp8_quantize_device(x.cuda(), pitch=2944)
     assert np.array_equal(q[:, :2880].cpu().numpy(), mxfp8.mx_quantize(x.numpy())[0]) and not q[:, 2880:].any()
 
