@@ -29,6 +29,9 @@ FLOPS_GATE_UP = 2.0 * T * TOPK * H * I * 2
 FLOPS_DOWN = 2.0 * T * TOPK * I * H
 FLOPS_TOTAL = FLOPS_GATE_UP + FLOPS_DOWN
 PEAK_FP8_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
+# HBM-side bytes of one gate/up launch: FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this script, each
+# scaled by what the same counter reads for a 1 GiB device copy (--copy-calibration): 2.0 and 1.0 KiB per unit.
+TRAFFIC_GATE_UP_BYTES = 1.127e9
 
 
 def make_inputs(dev, seed=0):
@@ -100,6 +103,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-pair", action="store_true", help="skip the linked vs one-unit paired timing")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a plain 1 GiB device copy, 10 times: the known-size kernel the FETCH_SIZE / "
+                         "WRITE_SIZE counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share of the routed-expert FFN; --gpus must be 1",
@@ -107,6 +113,14 @@ def main() -> int:
         return 2
 
     import torch
+    if args.copy_calibration:
+        src = torch.ones(1 << 30, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes_read": 1 << 30, "copy_calibration_bytes_written": 1 << 30, "launches": 10}))
+        return 0
     from pipelink_amd.host.backend import HipBackend
     from pipelink_amd.host.mok import MoKSession, code_pitch, scale_pitch
     from pipelink_amd.stages.mok import build as mok_build
@@ -181,7 +195,7 @@ def main() -> int:
         "roofline": {"bound": "mfma", "kernel": "pipelink_kernel (gate/up pass: grouped GEMM + SwiGLU + requant)",
                      "achieved": round(FLOPS_GATE_UP / (ms_gate_up * 1e-3) / 1e12, 2), "peak": PEAK_FP8_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(FLOPS_GATE_UP / (ms_gate_up * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4),
-                     "traffic": None, "launch_ms": round(ms_gate_up, 4),
+                     "traffic": TRAFFIC_GATE_UP_BYTES, "launch_ms": round(ms_gate_up, 4),
                      "down_pass": {"achieved": round(FLOPS_DOWN / (ms_down * 1e-3) / 1e12, 2), "launch_ms": round(ms_down, 4)}},
         "linked_over_one_unit": pair,
     }

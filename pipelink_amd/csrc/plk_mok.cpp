@@ -163,7 +163,6 @@ int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass,
   const int64_t max_tiles = max_row_tiles * fw.num_col_tiles;
   int64_t wgs = (int64_t)s->compute_units * s->link.workgroups_per_cu;
   if (wgs > max_tiles) wgs = max_tiles;
-  if (const char* dbg = getenv("PLK_MOK_DEBUG_GRID")) wgs = atoll(dbg);
   wgs = (wgs + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
   const uint32_t grid[3] = {(uint32_t)wgs, 1, 1};
   const uint32_t block[3] = {s->link.threads, 1, 1};

@@ -121,11 +121,11 @@ def test_stale_shared_declarations_are_refused(cell, tmp_path):
 
 
 def test_cli_prints_named_failures_and_exits_1(cell, tmp_path):
-    p = _mutated(cell[0], tmp_path, None, None, lambda pl: pl["exclusive"].append(["steady", "missing"]))
+    p = _mutated(cell[0], tmp_path, None, None, lambda pl: pl["exclusive"].append(["instr_gemm", "missing"]))
     proc = subprocess.run([sys.executable, "-m", "pipelink_amd.pipec", "link", str(p), "--out-dir", str(tmp_path / "o"),
                            "--plan-only"], capture_output=True, text=True, cwd=ROOT)
     assert proc.returncode == 1
-    assert proc.stderr.strip() == "pipec: [L-PHASE] $.pipeline.exclusive[0][1]: unknown phase"
+    assert proc.stderr.strip() == "pipec: [L-PHASE] $.pipeline.exclusive[1][1]: unknown phase"
     ok = subprocess.run([sys.executable, "-m", "pipelink_amd.pipec", "clauses", "--json"], capture_output=True, text=True, cwd=ROOT)
     assert ok.returncode == 0 and {"L-PROTO", "L-HANDLE", "L-PHASE"} <= {r["id"] for r in json.loads(ok.stdout)}
     ins = subprocess.run([sys.executable, "-m", "pipelink_amd.pipec", "inspect", str(cell[0] / "mok.gemm.plink")],
