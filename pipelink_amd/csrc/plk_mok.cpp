@@ -44,6 +44,14 @@ static int check_problem(const plk_mok_problem* p) {
     return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: code row pitch must be a multiple of 16 and at least K");
   if (p->num_tokens < 0 || p->routed_rows < 0)
     return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: negative row count");
+  {
+    // the kernel addresses one operand with 32-bit byte offsets from its base
+    const int64_t ldh = p->ld_q_h ? p->ld_q_h : p->hidden, ldi = p->ld_q_i ? p->ld_q_i : p->intermediate;
+    const int64_t lim = (int64_t)1 << 32;
+    if (p->num_tokens * ldh >= lim || p->routed_rows * ldi >= lim || (int64_t)p->intermediate * ldh >= lim ||
+        (int64_t)p->hidden * ldi >= lim)
+      return plk_hip_set_error(PLK_E_CAPACITY, "plk_mok: an operand (rows x row pitch) must stay below 4 GiB");
+  }
   if (p->routed_rows && (!p->x_q || !p->x_sc || !p->tokens_per_expert || !p->w_gate_q || !p->w_gate_sc ||
                          !p->w_up_q || !p->w_up_sc || !p->w_down_q || !p->w_down_sc || !p->hidden_q ||
                          !p->hidden_sc || !p->y))
@@ -78,7 +86,7 @@ int plk_mok_session_create(const void* image, size_t image_bytes, const plk_mok_
   for (auto& n : need)
     if (n[0] % 8 || n[0] + n[1] > link->params_bytes)
       return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_session_create: params entry outside the image or misaligned");
-  if (link->threads != 512) return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_session_create: image must use 512 threads");
+  if (link->threads != 256) return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_session_create: image must use 256 threads");
   auto* s = new plk_mok_session;
   s->link = *link;
   int rc = plk_hip_module_load(image, image_bytes, &s->module);

@@ -101,15 +101,16 @@ __device__ __forceinline__ void forward(const MokActResidue& p, const MokActTask
   const int chunk = lane & 7;
   const bool col_ok = t.col_begin + chunk * 16 < p.cols;  // column extents are multiples of 32
 #pragma unroll
-  for (int it = 0; it < TILE_X / 64; ++it) {
-    const int trow = wave * (TILE_X / 8) + it * 8 + (lane >> 3);
+  for (int it = 0; it < TILE_X / (THREADS / 64) / 8; ++it) {
+    const int trow = wave * (TILE_X / (THREADS / 64)) + it * 8 + (lane >> 3);
     const int row = t.row_begin + trow;
     if (row < t.row_end && col_ok) {
       const uint4 v = *reinterpret_cast<const uint4*>(stage + trow * STAGE_PITCH + chunk * 16);
       *reinterpret_cast<uint4*>(p.hidden_q + (int64_t)row * p.ld_q + t.col_begin + chunk * 16) = v;
     }
   }
-  if (tid < TILE_X) {
+  static_assert(THREADS == TILE_X, "one thread per routed row writes the row's scale bytes");
+  {
     const int row = t.row_begin + tid;
     if (row < t.row_end) {
       const uint32_t sc = *reinterpret_cast<const uint32_t*>(stage + STAGE_SCALE_OFF + tid * 4);

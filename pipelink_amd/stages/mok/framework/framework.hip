@@ -95,7 +95,7 @@ extern "C" __device__ void mok_framework_worker(const void* params, unsigned var
 
 PL_STAGE("mok.framework", "0.1.0");
 PL_PARAMS(MokFrameworkParams);
-PL_ROLE(worker, mok_framework_worker, 8);
+PL_ROLE(worker, mok_framework_worker, 4);
 PL_TOPOLOGY(true, "static");
 PL_VARIANT(0, {});
 PL_CALL(gemm_init, "mok_gemm_init", "extern \"C\" __device__ void pipelink_call_gemm_init(const void* view);");

@@ -9,22 +9,28 @@
 // four consecutive output columns of one routed row, which is what the requantising
 // epilogue and the bf16 store want.
 //
-// Ring: `depth` LDS slots of 65 KB.  A slot holds 128 contraction bytes of 256 routed rows
-// and of 256 weight rows, row-major (one 128-byte cache line per row), followed by one
-// dword of block scales (4 x e8m0) per weight row (weight scales are stored slot-major, so a
-// tile's 1 KB of them is one contiguous load).  The routed rows' scales are row-major in HBM
-// (rows are gathered); every fourth slot 16 bytes per row -- four slots' worth -- go to a
-// small double buffer behind the ring.  One global_load_lds_dwordx4 moves 8 rows:
-// eight lanes cover the 128 contiguous bytes of a row, so every L2 request is a full line.
-// The eight 16-byte chunks of a row are stored at position chunk ^ ((row / 2) % 8), which
-// makes a fragment read (32 consecutive rows, one chunk each) touch 16 different 16-byte
-// bank groups per 16 lanes.  The depth is a link-time handle; the ring offset inside the
-// workgroup's dynamic LDS is another.
+// Ring: `depth` LDS slots of 32 KB.  A slot holds 64 contraction bytes -- one MFMA step -- of
+// 256 routed rows and of 256 weight rows, row-major.  One global_load_lds_dwordx4 moves 16
+// rows: four lanes cover the 64 contiguous bytes of a row.  The four 16-byte chunks of a row
+// are stored at position chunk ^ ((row / 4) % 4), which makes a fragment read (16 lanes = 16
+// consecutive rows, one chunk each) touch 16 different 16-byte bank groups.  Behind the ring:
+// four 1 KB buffers of weight block scales (stored slot-major in HBM, one dword = 128
+// contraction bytes per row, so a tile's share is one contiguous load every second slot) and
+// two 4 KB buffers of routed-row scales (row-major in HBM because rows are gathered; 16 bytes
+// per row = eight slots' worth, fetched every eighth slot while the previous eight are in use).
+//
+// Schedule: one wave per SIMD, 128 x 128 outputs per wave in 256 accumulator registers.
+// While the 16 MFMAs of slot j run, the wave reads the operands of slot j+1 from LDS into a
+// second register set and the loads of slot j+depth are in flight, so neither the LDS latency
+// nor the L2 latency sits between two MFMAs.  One s_barrier per slot; it only waits for what
+// was issued a full slot earlier.  The depth is a link-time handle; the ring offset inside
+// the workgroup's dynamic LDS is another.
 #include <pipelink/stage.hpp>
 #ifndef PIPELINK_EMIT
+#include <type_traits>
 #include "../include/mok_device.hpp"
 
-extern "C" __device__ int pipelink_mok_gemm_depth();  // ring slots (2 or 3), bound at link time
+extern "C" __device__ int pipelink_mok_gemm_depth();  // ring slots (2 or 4), bound at link time
 extern "C" __device__ int pipelink_mok_gemm_arena();  // byte offset of the ring in dynamic LDS
 
 extern __shared__ __attribute__((aligned(1024))) unsigned char pipelink_smem[];
@@ -33,54 +39,70 @@ namespace mok_gemm_owner {
 using namespace mok;
 
 constexpr int WAVES = THREADS / 64;
-constexpr int X_GROUPS = TILE_X / 8 / WAVES;  // 8-row load groups per wave (4)
-constexpr int W_GROUPS = TILE_W / 8 / WAVES;  // (4)
-constexpr int LOADS_PER_SLOT = X_GROUPS + W_GROUPS + 2;  // upper bound: + weight scales + routed-row scales
+constexpr int X_GROUPS = TILE_X / 16 / WAVES;  // 16-row load groups per wave (4)
+constexpr int W_GROUPS = TILE_W / 16 / WAVES;  // (4)
+constexpr int TILE_LOADS = X_GROUPS + W_GROUPS;  // loads every wave issues for every slot, after the slot's scale loads
 
-// Addresses are a wave-uniform base (kept in scalar registers) plus a 32-bit lane offset: one
-// operand of one expert is far below 4 GiB, and 8 + 1 offsets cost half the vector registers
-// of 9 pointers.
+// Loads are buffer loads: a 128-bit resource (base address and byte extent, in scalar
+// registers), a 32-bit lane offset that is fixed for the tile, and the contraction offset as
+// the instruction's scalar offset -- no address arithmetic per load, and a read past the
+// extent returns zeros instead of faulting.  One operand of one expert is below 4 GiB (the
+// host checks).
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);  // raw, 32-bit data
+}
+// 16 (4) bytes per lane, buffer -> LDS; lane i lands at lds + 16*i (4*i)
+__device__ __forceinline__ void buf16_to_lds(rsrc_t r, uint32_t lane_off, uint32_t uni_off, unsigned char* lds) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lptr_t)lds, 16, (int)lane_off, (int)uni_off, 0, 0);
+}
+__device__ __forceinline__ void buf4_to_lds(rsrc_t r, uint32_t lane_off, uint32_t uni_off, unsigned char* lds) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lptr_t)lds, 4, (int)lane_off, (int)uni_off, 0, 0);
+}
+
 struct Loader {
-  const uint8_t* xbase;           // activations (all rows)
-  const uint8_t* wbase;           // this expert's weight matrix (gate or up or down, by wave)
-  const uint8_t* xscbase;         // routed rows' scales, row-major
-  const uint8_t* wscbase;         // this lane's 16 bytes (4 rows) of the tile's weight scales in slot 0
-  uint32_t wsc_slot_pitch;        // bytes between two slots of the weight scales
-  uint32_t xscsrc;                // this thread's routed row in the scale matrix (threads 0..255)
+  rsrc_t x;                       // activations (all rows)
+  rsrc_t w;                       // this expert's weight matrix (gate or up or down, by wave)
+  rsrc_t xsc;                     // routed rows' scales, row-major
+  rsrc_t wsc;                     // this expert's weight scales (gate or up or down, by wave), slot-major
+  uint32_t wsc_pair_pitch;        // bytes between two 128-byte pairs of the weight scales
+  uint32_t wscsrc;                // this thread's weight row: its dword of block scales
+  uint32_t xscsrc;                // this thread's routed row in the scale matrix
   uint32_t xsrc[X_GROUPS];        // this lane's 16 bytes of its row in each group, at k = 0
   uint32_t wsrc[W_GROUPS];
-  int chunk_byte;                 // byte offset inside the 128-byte line this lane fetches in even groups
   int xdst, wdst;                 // slot-relative LDS byte offsets of the wave's first group
 };
 
-__device__ __forceinline__ int swizzle(int row) { return (row >> 1) & 7; }
+__device__ __forceinline__ int swizzle(int row) { return (row >> 2) & 3; }
 
-// Issue one slot.  k_left = contraction bytes from this slot's start to the end of the row:
-// the last slot of a K that is not a multiple of 128 only fetches the chunks that exist.
-__device__ __forceinline__ void issue_slot(const Loader& ld, unsigned char* slot, unsigned char* xscale, int kbyte,
-                                           int k_left) {
-  // group j starts at tile row 8 * (4 * wave + j): odd groups flip bit 2 of the swizzle, so
-  // the lane's chunk there is the even-group chunk with bit 2 (64 bytes) flipped
+// Issue slot j into ring buffer `buf`.  Scale loads go first so that they are older than the
+// slot's tile loads: waiting until at most TILE_LOADS * m loads are outstanding then covers
+// every load of all but the youngest m slots, whatever scale loads those carried.
+// J8 is j % 8 where the caller knows it at compile time, else -1.
+template <int J8 = -1>
+__device__ __forceinline__ void issue_slot(const Loader& ld, unsigned char* ring, unsigned char* wscale,
+                                           unsigned char* xscale, int j, int buf) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t kbyte = (uint32_t)j * K_SLOT;
+  const int j8 = J8 >= 0 ? J8 : (j & 7);
+  unsigned char* slot = ring + buf * SLOT_BYTES;
+  // every eighth slot: 16 scale bytes of each routed row (this slot and the next seven)
+  if (j8 == 0) buf16_to_lds(ld.xsc, ld.xscsrc, kbyte >> 5, xscale + ((j >> 3) & 1) * (TILE_X * 16) + wave * 1024);
+  // every second slot: the tile's weight scales of this pair, one row per thread
+  if ((j8 & 1) == 0)
+    buf4_to_lds(ld.wsc, ld.wscsrc, (uint32_t)(j >> 1) * ld.wsc_pair_pitch, wscale + (j8 >> 1) * (TILE_W * 4) + wave * 256);
 #pragma unroll
-  for (int j = 0; j < X_GROUPS; ++j)
-    if ((ld.chunk_byte ^ ((j & 1) << 6)) < k_left) load16_to_lds(ld.xbase + kbyte + ld.xsrc[j], slot + ld.xdst + j * 1024);
+  for (int i = 0; i < X_GROUPS; ++i) buf16_to_lds(ld.x, ld.xsrc[i], kbyte, slot + ld.xdst + i * 1024);
 #pragma unroll
-  for (int j = 0; j < W_GROUPS; ++j)
-    if ((ld.chunk_byte ^ ((j & 1) << 6)) < k_left) load16_to_lds(ld.wbase + kbyte + ld.wsrc[j], slot + ld.wdst + j * 1024);
-  const int wave = threadIdx.x >> 6;
-  const int s = kbyte >> 7;  // slot index
-  // wave 4: the tile's weight scales of this slot, 4 rows per lane
-  if (wave == 4) load16_to_lds(ld.wscbase + (size_t)s * ld.wsc_slot_pitch, slot + SLOT_X_BYTES + SLOT_W_BYTES);
-  // waves 0-3, every fourth slot: 16 scale bytes of each routed row (this slot and the next three)
-  if (wave < 4 && (s & 3) == 0) load16_to_lds(ld.xscbase + (kbyte >> 5) + ld.xscsrc, xscale + ((s >> 2) & 1) * (TILE_X * 16) + wave * 1024);
+  for (int i = 0; i < W_GROUPS; ++i) buf16_to_lds(ld.w, ld.wsrc[i], kbyte, slot + ld.wdst + i * 1024);
 }
 
 // MFMA 32x32x64 f8f6f4 operand of lane (row = lane % 32, half = lane / 32): registers 0-3
 // hold 16 bytes of the step's first 32-element block, registers 4-7 16 bytes of its second
 // block; the scale of block 0 is taken from lanes 0-31 and that of block 1 from lanes 32-63
-// (measured on gfx950 with a one-instruction probe).  So in 64-byte step s of a slot a lane
-// reads chunks 4s + half and 4s + half + 2 of its row; with the XOR swizzle these are the
-// step-0 offsets with bit 6 (step) and bit 5 (second block) flipped.
+// (measured on gfx950 with a one-instruction probe).  So a lane reads chunks half and
+// half + 2 of its row; with the XOR swizzle the second is the first with bit 5 flipped.
 __device__ __forceinline__ v8i read_frag(const unsigned char* slot, int off) {
   const v4i lo = *reinterpret_cast<const v4i*>(slot + off);
   const v4i hi = *reinterpret_cast<const v4i*>(slot + (off ^ 32));
@@ -99,92 +121,119 @@ __device__ __forceinline__ void wg_barrier() {
   asm volatile("" ::: "memory");
 }
 
+// wait until at most N global loads are outstanding and every LDS read has returned
 template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
+__device__ __forceinline__ void wait_loads_and_reads() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
-  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
+  __builtin_amdgcn_s_waitcnt(0x0070 | (N & 0xF) | ((N >> 4) << 14));
+}
+
+struct Operands {
+  v8i x[XFRAGS], w[WFRAGS];
+};
+
+__device__ __forceinline__ void read_operands(Operands& o, const unsigned char* slot, const int (&xoff)[XFRAGS],
+                                              const int (&woff)[WFRAGS]) {
+#pragma unroll
+  for (int b = 0; b < XFRAGS; ++b) o.x[b] = read_frag(slot, xoff[b]);
+#pragma unroll
+  for (int a = 0; a < WFRAGS; ++a) o.w[a] = read_frag(slot, woff[a]);
+}
+
+// Block scales of the 128-byte pair that starts at slot j (j even): one dword per row; lanes
+// of the upper half use blocks 1 and 3, shifted down into bytes 0 and 2 where the MFMA's
+// op_sel picks them (0 in the pair's first slot, 2 in its second).  The routed rows' dwords
+// sit 16 bytes apart (a 4-way bank conflict on four small reads per pair).
+template <int J8 = -1>
+__device__ __forceinline__ void read_scales(int (&sx)[XFRAGS], int (&sw)[WFRAGS], const unsigned char* wscale,
+                                            const unsigned char* xscale, int j, const int (&xscoff)[XFRAGS],
+                                            const int (&wscoff)[WFRAGS], int half) {
+  const int c = (J8 >= 0 ? J8 : (j & 7)) >> 1;
+  const unsigned char* xbuf = xscale + ((j >> 3) & 1) * (TILE_X * 16);
+#pragma unroll
+  for (int b = 0; b < XFRAGS; ++b)
+    sx[b] = (int)(*reinterpret_cast<const uint32_t*>(xbuf + 4 * c + xscoff[b]) >> (8 * half));
+  const unsigned char* wbuf = wscale + c * (TILE_W * 4);
+#pragma unroll
+  for (int a = 0; a < WFRAGS; ++a) sw[a] = (int)(*reinterpret_cast<const uint32_t*>(wbuf + wscoff[a]) >> (8 * half));
 }
 
 template <bool ODD>
-__device__ __forceinline__ void mma_step(const unsigned char* slot, const int (&xoff)[XFRAGS],
-                                         const int (&woff)[WFRAGS], const int (&sx)[XFRAGS],
-                                         const int (&sw)[WFRAGS], AccFrag& acc) {
-  v8i xf[XFRAGS], wf[WFRAGS];
-#pragma unroll
-  for (int b = 0; b < XFRAGS; ++b) xf[b] = read_frag(slot, xoff[b] ^ (ODD ? 64 : 0));
-#pragma unroll
-  for (int a = 0; a < WFRAGS; ++a) wf[a] = read_frag(slot, woff[a] ^ (ODD ? 64 : 0));
+__device__ __forceinline__ void mma_step(const Operands& o, const int (&sx)[XFRAGS], const int (&sw)[WFRAGS],
+                                         AccFrag& acc) {
 #pragma unroll
   for (int a = 0; a < WFRAGS; ++a)
 #pragma unroll
     for (int b = 0; b < XFRAGS; ++b)
-      acc.v[a][b] = ODD ? __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[a], xf[b], acc.v[a][b], 0, 0, 2, sw[a], 2, sx[b])
-                        : __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[a], xf[b], acc.v[a][b], 0, 0, 0, sw[a], 0, sx[b]);
+      acc.v[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.w[a], o.x[b], acc.v[a][b], 0, 0, ODD ? 2 : 0,
+                                                                    sw[a], ODD ? 2 : 0, sx[b]);
 }
 
 template <int DEPTH>
 __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmTask& t, AccFrag& acc) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: resources chosen by it stay scalar
   const int r32 = lane & 31;
   const int half = lane >> 5;
   const bool gate_up = t.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
+  const int expert = __builtin_amdgcn_readfirstlane(t.expert);
   const MokMxView& act = gate_up ? g.x : g.hidden;
-  const int K = act.k;
-  const int nslots = (K + K_SLOT - 1) / K_SLOT;
+  const int n = act.k / K_SLOT;  // the host rejects a contraction length that is not a multiple of 64
   unsigned char* ring = pipelink_smem + pipelink_mok_gemm_arena();
-  unsigned char* xscale = ring + DEPTH * SLOT_BYTES;  // routed-row scale double buffer behind the ring
+  unsigned char* wscale = ring + DEPTH * SLOT_BYTES;
+  unsigned char* xscale = wscale + WSCALE_BYTES;
 
   // ---- loader addresses (fixed for the tile) ---------------------------------------
-  // lane -> (row lane/8 of an 8-row group, LDS position lane%8); it fetches the chunk that
-  // belongs at that position
+  // lane -> (row lane/4 of a 16-row group, LDS position lane%4); it fetches the chunk that
+  // belongs at that position.  Groups start at multiples of 16 rows, so the swizzle of a row
+  // only depends on its place in the group.
   Loader ld;
   {
-    const int lrow = lane >> 3;
-    const int pos = lane & 7;
-    ld.chunk_byte = 16 * (pos ^ swizzle(lrow));
-    static_assert(X_GROUPS % 2 == 0 && W_GROUPS % 2 == 0, "a wave's first group must start at a multiple of 16 rows");
+    const int lrow = lane >> 2;
+    const int chunk = 16 * ((lane & 3) ^ swizzle(lrow));
 #pragma unroll
-    for (int j = 0; j < X_GROUPS; ++j) {
-      const int trow = (wave * X_GROUPS + j) * 8 + lrow;  // tile-local routed row
+    for (int i = 0; i < X_GROUPS; ++i) {
+      const int trow = (wave * X_GROUPS + i) * 16 + lrow;  // tile-local routed row
       int row = t.row_begin + trow;
       row = row < t.row_end ? row : t.row_end - 1;
       const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
-      ld.xsrc[j] = (uint32_t)src * (uint32_t)act.ld_q + 16 * (pos ^ swizzle(trow));
+      ld.xsrc[i] = (uint32_t)src * (uint32_t)act.ld_q + chunk;
     }
-    ld.xbase = act.q;
+    ld.x = make_rsrc(act.q, (uint32_t)act.rows * (uint32_t)act.ld_q);
     ld.xdst = wave * X_GROUPS * 1024;
     const MokMxView& wv = gate_up ? (wave < WAVES / 2 ? g.w_gate : g.w_up) : g.w_down;
 #pragma unroll
-    for (int j = 0; j < W_GROUPS; ++j) {
-      const int wl = (wave * W_GROUPS + j) * 8 + lrow;  // tile-local weight row
+    for (int i = 0; i < W_GROUPS; ++i) {
+      const int wl = (wave * W_GROUPS + i) * 16 + lrow;  // tile-local weight row
       int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
       col = col < wv.rows ? col : wv.rows - 1;
-      ld.wsrc[j] = (uint32_t)col * (uint32_t)wv.ld_q + 16 * (pos ^ swizzle(wl));
+      ld.wsrc[i] = (uint32_t)col * (uint32_t)wv.ld_q + chunk;
     }
-    ld.wbase = wv.q + (int64_t)t.expert * wv.expert_pitch_q;
+    ld.w = make_rsrc(wv.q + (int64_t)expert * wv.expert_pitch_q, (uint32_t)wv.rows * (uint32_t)wv.ld_q);
     ld.wdst = SLOT_X_BYTES + wave * W_GROUPS * 1024;
-    // routed-row scales: thread tid < 256 fetches row tid's 16-byte piece
+    // routed-row scales: thread tid fetches row tid's 16-byte piece
     {
-      int row = t.row_begin + (tid & (TILE_X - 1));
+      int row = t.row_begin + tid;
       row = row < t.row_end ? row : t.row_end - 1;
       const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
-      ld.xscbase = act.sc;
+      ld.xsc = make_rsrc(act.sc, (uint32_t)act.rows * (uint32_t)act.ld_sc);
       ld.xscsrc = (uint32_t)src * (uint32_t)act.ld_sc;
     }
-    // weight scales, slot-major [slot][row][4]: lane l of one wave fetches tile rows 4l .. 4l+3
+    // weight scales, slot-major [pair][row][4]: thread tid fetches tile row tid's dword
     {
-      const int wl = 4 * lane;
-      const MokMxView& sv = gate_up ? (wl < TILE_W / 2 ? g.w_gate : g.w_up) : g.w_down;
-      int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
-      col = col <= sv.rows - 4 ? col : sv.rows - 4;  // row counts are multiples of 32
-      ld.wscbase = sv.sc + (int64_t)t.expert * sv.expert_pitch_sc + (int64_t)col * 4;
-      ld.wsc_slot_pitch = (uint32_t)sv.rows * 4u;
+      static_assert(THREADS == TILE_W, "one thread per weight row");
+      const MokMxView& sv = gate_up ? (wave < WAVES / 2 ? g.w_gate : g.w_up) : g.w_down;
+      int col = t.col_begin + (gate_up ? (tid & (TILE_W / 2 - 1)) : tid);
+      col = col < sv.rows ? col : sv.rows - 1;
+      ld.wsc = make_rsrc(sv.sc + (int64_t)expert * sv.expert_pitch_sc,
+                         (uint32_t)((sv.k + K_PAIR - 1) / K_PAIR) * (uint32_t)sv.rows * 4u);
+      ld.wscsrc = (uint32_t)col * 4u;
+      ld.wsc_pair_pitch = (uint32_t)sv.rows * 4u;
     }
   }
 
-  // ---- per-fragment LDS read offsets (step 0, first block) ---------------------------
+  // ---- per-fragment LDS read offsets (first block) ------------------------------------
   int xoff[XFRAGS], woff[WFRAGS], xscoff[XFRAGS], wscoff[WFRAGS];
 #pragma unroll
   for (int b = 0; b < XFRAGS; ++b) {
@@ -196,7 +245,7 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   for (int a = 0; a < WFRAGS; ++a) {
     const int wl = wrow0(wave, a) + r32;
     woff[a] = SLOT_X_BYTES + wl * K_SLOT + 16 * (half ^ swizzle(wl));
-    wscoff[a] = SLOT_X_BYTES + SLOT_W_BYTES + wl * 4;
+    wscoff[a] = wl * 4;
   }
 
 #pragma unroll
@@ -206,44 +255,109 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc.v[a][b][r] = 0.0f;
 
-  // ---- prologue: fill depth-1 slots ---------------------------------------------------
+  // ---- prologue: fill the ring, fetch slot 0's operands --------------------------------
 #pragma unroll
-  for (int s = 0; s < DEPTH - 1; ++s)
-    if (s < nslots) issue_slot(ld, ring + s * SLOT_BYTES, xscale, s * K_SLOT, K - s * K_SLOT);
+  for (int s = 0; s < DEPTH; ++s)
+    if (s < n) issue_slot(ld, ring, wscale, xscale, s, s);
+  if (n >= DEPTH)
+    wait_loads_and_reads<TILE_LOADS * (DEPTH - 1)>();
+  else
+    wait_loads_and_reads<0>();
+  wg_barrier();
+  Operands even, odd;
+  int sx[XFRAGS], sw[WFRAGS], sxn[XFRAGS], swn[WFRAGS];
+  read_operands(even, ring, xoff, woff);
+  read_scales(sx, sw, wscale, xscale, 0, xscoff, wscoff, half);
 
-  int cur = 0;           // slot the next iteration consumes
-  int fill = DEPTH - 1;  // slot the next issued load fills
-  for (int i = 0; i < nslots; ++i) {
-    // loads younger than slot i's: the slots i+1 .. i+DEPTH-2
-    if (i + DEPTH - 2 < nslots)
-      wait_vmcnt<(DEPTH - 2) * LOADS_PER_SLOT>();
-    else
-      wait_vmcnt<0>();
-    wg_barrier();  // slot i has landed for every wave; everyone is done reading slot i-1
-    if (i + DEPTH - 1 < nslots)
-      issue_slot(ld, ring + fill * SLOT_BYTES, xscale, (i + DEPTH - 1) * K_SLOT, K - (i + DEPTH - 1) * K_SLOT);
-    fill = fill + 1 == DEPTH ? 0 : fill + 1;
-    const unsigned char* slot = ring + cur * SLOT_BYTES;
-    cur = cur + 1 == DEPTH ? 0 : cur + 1;
-
-    // block scales of the slot: lanes of the upper half use blocks 1 and 3, shifted down
-    // into bytes 0 and 2 where the MFMA's op_sel picks them
-    int sx[XFRAGS], sw[WFRAGS];
+  // Step j multiplies slot j (already in registers) while it fetches slot j+1's operands from
+  // LDS; the barrier in front says slot j+1 has landed for every wave and every wave holds
+  // slot j in registers, so slot j's buffer takes the loads of slot j+DEPTH.
+  //
+  // Steady state: groups of eight steps, fully unrolled, as long as every step of the group
+  // still has a slot to issue.  Ring buffer, scale buffer, scale byte and the slots that carry
+  // scale loads are compile-time constants there, so the group is one basic block and the
+  // MFMAs stay where they are written, between the LDS reads they overlap with.
+  static_assert(8 % DEPTH == 0, "a group of eight slots must start at ring buffer 0");
+  int j = 0;
+  for (; j + 8 + DEPTH <= n; j += 8) {
+    auto step = [&](auto S_) {
+      constexpr int S = decltype(S_)::value;
+      constexpr bool ODD = S & 1;
+      Operands& cur = ODD ? odd : even;
+      Operands& next = ODD ? even : odd;
+      __builtin_amdgcn_sched_barrier(0);  // nothing of the previous step sinks below, nothing of this one rises above
+      wait_loads_and_reads<TILE_LOADS * (DEPTH - 2)>();  // loads younger than slot j+S+1's: DEPTH-2 slots
+      wg_barrier();
+      issue_slot<(S + DEPTH) & 7>(ld, ring, wscale, xscale, j + S + DEPTH, S % DEPTH);
+      read_operands(next, ring + ((S + 1) % DEPTH) * SLOT_BYTES, xoff, woff);
+      if (ODD) read_scales<(S + 1) & 7>(sxn, swn, wscale, xscale, j + S + 1, xscoff, wscoff, half);
+      mma_step<ODD>(cur, sx, sw, acc);
+      // issue order inside the step: an MFMA first (the pipe must not drain behind the
+      // barrier), the global loads spread over the first eight MFMAs, the LDS reads over the rest
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x010, 3, 0);  // VMEM: the scale loads and the first tile load
 #pragma unroll
-    for (int b = 0; b < XFRAGS; ++b)
-      sx[b] = (int)(*reinterpret_cast<const uint32_t*>(xscale + ((i >> 2) & 1) * (TILE_X * 16) + xscoff[b] + 4 * (i & 3)) >> (8 * half));
+      for (int i = 1; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);  // VMEM
+      }
 #pragma unroll
-    for (int a = 0; a < WFRAGS; ++a) sw[a] = (int)(*reinterpret_cast<const uint32_t*>(slot + wscoff[a]) >> (8 * half));
-    mma_step<false>(slot, xoff, woff, sx, sw, acc);
-    if (K - i * K_SLOT > 64) mma_step<true>(slot, xoff, woff, sx, sw, acc);
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);  // LDS reads
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (ODD) {
+#pragma unroll
+        for (int b = 0; b < XFRAGS; ++b) sx[b] = sxn[b];
+#pragma unroll
+        for (int a = 0; a < WFRAGS; ++a) sw[a] = swn[a];
+      }
+    };
+    step(std::integral_constant<int, 0>{});
+    step(std::integral_constant<int, 1>{});
+    step(std::integral_constant<int, 2>{});
+    step(std::integral_constant<int, 3>{});
+    step(std::integral_constant<int, 4>{});
+    step(std::integral_constant<int, 5>{});
+    step(std::integral_constant<int, 6>{});
+    step(std::integral_constant<int, 7>{});
   }
-  wg_barrier();  // ring free for the next tile
+
+  // Remaining slots (fewer than 8 + DEPTH), same steps with run-time slot numbers.  The MFMA
+  // chain is straight-line code: past the last slot `advance` still runs (it reads a buffer
+  // nobody uses), which keeps control flow out of the accumulator's live range.
+  int buf = 0;  // ring buffer of slot j (j is a multiple of 8 here)
+  auto advance = [&](int jj, Operands& next) {
+    // loads younger than slot jj+1's: slots jj+2 .. jj+DEPTH-1, if all of those exist
+    if (jj + DEPTH <= n)
+      wait_loads_and_reads<TILE_LOADS * (DEPTH - 2)>();
+    else
+      wait_loads_and_reads<0>();
+    wg_barrier();
+    if (jj + DEPTH < n) issue_slot(ld, ring, wscale, xscale, jj + DEPTH, buf);
+    buf = buf + 1 == DEPTH ? 0 : buf + 1;
+    read_operands(next, ring + buf * SLOT_BYTES, xoff, woff);
+  };
+  for (; j + 1 < n; j += 2) {
+    advance(j, odd);
+    mma_step<false>(even, sx, sw, acc);
+    advance(j + 1, even);
+    read_scales(sxn, swn, wscale, xscale, j + 2, xscoff, wscoff, half);
+    mma_step<true>(odd, sx, sw, acc);
+#pragma unroll
+    for (int b = 0; b < XFRAGS; ++b) sx[b] = sxn[b];
+#pragma unroll
+    for (int a = 0; a < WFRAGS; ++a) sw[a] = swn[a];
+  }
+  if (n & 1) mma_step<false>(even, sx, sw, acc);  // a last single slot is already in registers
+  wg_barrier();  // every wave holds its last operands in registers: the ring is free
 }
 
 // bf16 epilogue of the down op.  The accumulator is transposed through the (now idle) ring so
-// that the global stores are 16 bytes per lane and 512 contiguous bytes per routed row.
+// that the global stores are 16 bytes per lane and 512 contiguous bytes per routed row.  A
+// ring too small for the whole tile stages the two 128-row halves one after the other.
 constexpr int Y_PITCH = TILE_W * 2 + 16;  // bytes per staged row: 256 bf16 + pad against bank conflicts
-static_assert(TILE_X * Y_PITCH <= 2 * SLOT_BYTES + XSCALE_BYTES, "staging tile must fit the two-slot ring");
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -253,38 +367,54 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // v_cvt_pk_bf16_f32, nearest even
 }
 
+template <int DEPTH>
 __device__ __forceinline__ void store_down(const MokGemmResidue& g, const MokGemmTask& t, const AccFrag& acc) {
+  constexpr int RING_BYTES = DEPTH * SLOT_BYTES + WSCALE_BYTES + XSCALE_BYTES;
+  constexpr int PASSES = TILE_X * Y_PITCH <= RING_BYTES ? 1 : 2;
+  constexpr int ROWS = TILE_X / PASSES;  // rows staged per pass
+  static_assert(ROWS * Y_PITCH <= RING_BYTES, "half a tile must fit the ring");
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   unsigned char* stage = pipelink_smem + pipelink_mok_gemm_arena();
+  const int chunk = lane & 31;                                  // 8 columns = 16 bytes
+  const bool col_ok = t.col_begin + chunk * 8 < g.w_down.rows;  // column extents are multiples of 32
 #pragma unroll
-  for (int b = 0; b < XFRAGS; ++b) {
-    unsigned char* rowp = stage + (xrow0(wave, b) + (lane & 31)) * Y_PITCH;
+  for (int pass = 0; pass < PASSES; ++pass) {
+    if (PASSES == 1 || wave_x(wave) == pass) {
 #pragma unroll
-    for (int a = 0; a < WFRAGS; ++a) {
+      for (int b = 0; b < XFRAGS; ++b) {
+        unsigned char* rowp = stage + (xrow0(wave, b) - pass * ROWS + (lane & 31)) * Y_PITCH;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int col = wrow0(wave, a) + 8 * q + 4 * (lane >> 5);
-        uint2 pk;
-        pk.x = pack_bf16x2(acc.v[a][b][4 * q + 0], acc.v[a][b][4 * q + 1]);
-        pk.y = pack_bf16x2(acc.v[a][b][4 * q + 2], acc.v[a][b][4 * q + 3]);
-        *reinterpret_cast<uint2*>(rowp + col * 2) = pk;
+        for (int a = 0; a < WFRAGS; ++a) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int col = wrow0(wave, a) + 8 * q + 4 * (lane >> 5);
+            uint2 pk;
+            pk.x = pack_bf16x2(acc.v[a][b][4 * q + 0], acc.v[a][b][4 * q + 1]);
+            pk.y = pack_bf16x2(acc.v[a][b][4 * q + 2], acc.v[a][b][4 * q + 3]);
+            *reinterpret_cast<uint2*>(rowp + col * 2) = pk;
+          }
+        }
       }
     }
-  }
-  __syncthreads();
-  const int chunk = lane & 31;                              // 8 columns = 16 bytes
-  const bool col_ok = t.col_begin + chunk * 8 < g.w_down.rows;  // column extents are multiples of 32
+    __syncthreads();
 #pragma unroll 4
-  for (int it = 0; it < TILE_X / 16; ++it) {
-    const int trow = wave * (TILE_X / 8) + it * 2 + (lane >> 5);
-    const int row = t.row_begin + trow;
-    if (row < t.row_end && col_ok) {
-      const uint4 v = *reinterpret_cast<const uint4*>(stage + trow * Y_PITCH + chunk * 16);
-      *reinterpret_cast<uint4*>(g.y + (int64_t)row * g.ld_y + t.col_begin + chunk * 8) = v;
+    for (int it = 0; it < ROWS / WAVES / 2; ++it) {
+      const int srow = wave * (ROWS / WAVES) + it * 2 + (lane >> 5);
+      const int row = t.row_begin + pass * ROWS + srow;
+      if (row < t.row_end && col_ok) {
+        const uint4 v = *reinterpret_cast<const uint4*>(stage + srow * Y_PITCH + chunk * 16);
+        *reinterpret_cast<uint4*>(g.y + (int64_t)row * g.ld_y + t.col_begin + chunk * 8) = v;
+      }
     }
+    __syncthreads();  // the ring is reused by the next pass or the next tile's loads
   }
-  __syncthreads();  // the ring is reused by the next tile's loads
+}
+
+template <int DEPTH>
+__device__ __forceinline__ void run(const MokGemmResidue& g, const MokGemmTask& t, AccFrag& acc) {
+  mainloop<DEPTH>(g, t, acc);
+  if (t.op == MOK_GEMM_FWD_ROUTED_DOWN) store_down<DEPTH>(g, t, acc);
 }
 
 }  // namespace mok_gemm_owner
@@ -298,11 +428,10 @@ extern "C" __device__ void mok_gemm_fwd(const void* view, const MokGemmTask* tas
   (void)counters;
   (void)phase;
   const auto& g = *static_cast<const MokGemmResidue*>(static_cast<const pipelink_host_view*>(view)->residue);
-  if (pipelink_mok_gemm_depth() == 2)
-    mok_gemm_owner::mainloop<2>(g, *task, *acc);
-  else
-    mok_gemm_owner::mainloop<3>(g, *task, *acc);  // needs 3 x 66 KB: beyond one CU's LDS at this tile size
-  if (task->op == MOK_GEMM_FWD_ROUTED_DOWN) mok_gemm_owner::store_down(g, *task, *acc);
+  switch (pipelink_mok_gemm_depth()) {  // a link-time constant: one case survives
+    case 2: mok_gemm_owner::run<2>(g, *task, *acc); break;
+    default: mok_gemm_owner::run<4>(g, *task, *acc); break;
+  }
 }
 #else  // PIPELINK_EMIT: host-evaluated annotations only
 #include "../include/mok_abi.h"
@@ -318,14 +447,14 @@ PL_EXPORT(mok_gemm_fwd, mok_gemm_fwd,
           "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc);");
 PL_SERVE(gemm_init, "mok_gemm_init");
 PL_SERVE(gemm_fwd, "mok_gemm_fwd");
-// ring of `depth` slots: 256 x 128 B of routed rows, 256 x 128 B of weight rows, 1 KB of weight scales
-// + 8 KB behind the ring: double buffer of the routed rows' scales
-PL_CLAIM_RING("pipelink_mok_gemm_arena", "smem", 8192, "pipelink_mok_gemm_depth", 66560, 1024, "phase:instr_gemm");
+// ring of `depth` slots: 256 x 64 B of routed rows, 256 x 64 B of weight rows
+// + 12 KB behind the ring: four 1 KB buffers of weight scales, two 4 KB buffers of routed-row scales
+PL_CLAIM_RING("pipelink_mok_gemm_arena", "smem", 12288, "pipelink_mok_gemm_depth", 32768, 1024, "phase:instr_gemm");
 PL_USES("pipelink_mok_gemm_depth");
 PL_USES("pipelink_mok_gemm_arena");
 PL_FACT("mok.gemm.TILE_X", 256);
 PL_FACT("mok.gemm.TILE_W", 256);
-PL_FACT("mok.gemm.K_SLOT", 128);
+PL_FACT("mok.gemm.K_SLOT", 64);
 PL_PRELUDE("../include/mok_abi.h");
 PL_PRELUDE("../include/mok_device.hpp");
 PL_EMIT_MAIN()

@@ -15,21 +15,22 @@ typedef int v2i __attribute__((ext_vector_type(2)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 // ---- tile geometry published by the GEMM owner (facts mok.gemm.*) -------------------
-// One workgroup tile = TILE_X routed rows x TILE_W weight rows, 8 waves as 4 (rows) x 2
-// (weights), each wave a 64 x 128 sub-tile.  For the gate/up op the weight rows are
-// TILE_W/2 gate columns followed by the same TILE_W/2 up columns, so gate and up of one
-// output element meet in one register.
+// One workgroup tile = TILE_X routed rows x TILE_W weight rows, 4 waves (one per SIMD) as
+// 2 (rows) x 2 (weights), each wave a 128 x 128 sub-tile.  For the gate/up op the weight
+// rows are TILE_W/2 gate columns followed by the same TILE_W/2 up columns, so gate and up of
+// one output element meet in one lane.
 constexpr int TILE_X = 256;
 constexpr int TILE_W = 256;
-constexpr int K_SLOT = 128;     // contraction bytes per ring slot = two MFMA 32x32x64 steps
+constexpr int K_SLOT = 64;      // contraction bytes per ring slot = one MFMA 32x32x64 step
+constexpr int K_PAIR = 128;     // contraction bytes one dword of four e8m0 block scales covers
 constexpr int WFRAGS = 4;       // 32-row weight fragments per wave
-constexpr int XFRAGS = 2;       // 32-row activation fragments per wave
-constexpr int THREADS = 512;
+constexpr int XFRAGS = 4;       // 32-row activation fragments per wave
+constexpr int THREADS = 256;
 constexpr int SLOT_X_BYTES = TILE_X * K_SLOT;
 constexpr int SLOT_W_BYTES = TILE_W * K_SLOT;
-constexpr int SLOT_SCALE_BYTES = TILE_W * 4;             // one dword (4 block scales) per weight row
-constexpr int SLOT_BYTES = SLOT_X_BYTES + SLOT_W_BYTES + SLOT_SCALE_BYTES;  // 66560
-constexpr int XSCALE_BYTES = 2 * TILE_X * 16;            // two buffers of 16 scale bytes (4 slots) per routed row
+constexpr int SLOT_BYTES = SLOT_X_BYTES + SLOT_W_BYTES;  // 32768
+constexpr int WSCALE_BYTES = 4 * TILE_W * 4;             // four buffers of one dword (4 block scales) per weight row
+constexpr int XSCALE_BYTES = 2 * TILE_X * 16;            // two buffers of 16 scale bytes (8 slots) per routed row
 
 // fp32 accumulator of one wave: [weight fragment][row fragment] MFMA 32x32 C tiles.
 // Element (reg r, lane l) of tile (a, b) is
@@ -46,7 +47,7 @@ __device__ __forceinline__ int wave_x(int wave) { return wave >> 1; }
 __device__ __forceinline__ int wrow0(int wave, int a) {
   return (a < 2 ? 0 : TILE_W / 2) + wave_w(wave) * 64 + (a & 1) * 32;
 }
-__device__ __forceinline__ int xrow0(int wave, int b) { return wave_x(wave) * 64 + b * 32; }
+__device__ __forceinline__ int xrow0(int wave, int b) { return wave_x(wave) * 128 + b * 32; }
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;

@@ -31,16 +31,16 @@ def cell(tmp_path_factory):
 def test_link_json_records_the_solved_cell(cell):
     out, res = cell
     link = json.loads((out / "link" / "link.json").read_text())
-    assert link["kernel_symbol"] == "pipelink_kernel" and link["threads"] == 512
-    # three 65 KB slots do not fit 160 KB of LDS: the solver falls back to the largest depth that does
-    assert link["bindings"]["pipelink_mok_gemm_depth"] == [2, "solved"]
-    assert link["dyn_smem_bytes"] == 2 * 66560 + 8192 + 2056 <= 160 * 1024
+    assert link["kernel_symbol"] == "pipelink_kernel" and link["threads"] == 256
+    # four 32 KB slots + 12 KB of scale buffers + the schedule table fit 160 KB of LDS: the preferred depth is taken
+    assert link["bindings"]["pipelink_mok_gemm_depth"] == [4, "solved"]
+    assert link["dyn_smem_bytes"] == 4 * 32768 + 12288 + 2056 <= 160 * 1024
     assert [e["stage_id"] for e in link["params"]["entries"]] == ["mok.framework", "mok.gemm", "mok.act"]
     assert link["params"]["total_bytes"] == 344
     assert {e["channel"] for e in link["protocol_expansions"]} == {"gemm_init", "gemm_fwd", "act_init", "act_fwd"}
     obs = link["observed"]
     assert obs["calls"] == 0 and obs["private_segment_fixed_size"] <= 64 and obs["mfma"] >= 16   # a few spilled dwords at most
-    assert obs["vgpr_count"] <= link["regs_cap"] == 256
+    assert obs["vgpr_count"] <= link["regs_cap"] == 512
     assert link["facts"]["mok.gemm.TILE_X"] == 256
     assert set(link["input_hashes"]) == {"mok.framework", "mok.gemm", "mok.act"}
 
@@ -62,7 +62,8 @@ def _mutated(cell_dir: Path, tmp_path: Path, stage_id: str | None, mutate, pipel
 
 
 def test_forced_depth_beyond_lds_is_l_overlap(cell, tmp_path):
-    p = _mutated(cell[0], tmp_path, None, None, lambda pl: pl["forced_bindings"].update(pipelink_mok_gemm_depth=3))
+    p = _mutated(cell[0], tmp_path, None, None, lambda pl: (pl["handles"]["pipelink_mok_gemm_depth"]["values"].insert(0, 6),
+                                                       pl["forced_bindings"].update(pipelink_mok_gemm_depth=6)))
     with pytest.raises(SolveError) as err:
         linker.link(p, tmp_path / "link", codegen=False)
     assert err.value.clause_ids == {"L-OVERLAP"}
@@ -175,7 +176,7 @@ def test_hostless_launcher_params_contract(cell):
     blob = be.mem[s.params_addr]
     assert blob[0:40] == b"\x01" * 40 and blob[40:304] == b"\x02" * 264 and blob[304:344] == b"\x03" * 40
     s.launch()
-    assert be.launches == [(s.params_addr, (16, 1, 1), (512, 1, 1), link["dyn_smem_bytes"])]
+    assert be.launches == [(s.params_addr, (16, 1, 1), (256, 1, 1), link["dyn_smem_bytes"])]
     assert s.read("a").tolist() == [0, 1, 2, 3] and s.read("b").tolist() == [0.0] * 8
     s.write("b", np.ones(8, np.float32))
     assert s.read("b").sum() == 8
