@@ -9,11 +9,16 @@
 // four consecutive output columns of one routed row, which is what the requantising
 // epilogue and the bf16 store want.
 //
-// Ring: `depth` LDS slots of 32 KB.  A slot holds 64 contraction bytes -- one MFMA step -- of
-// 256 routed rows and of 256 weight rows, row-major.  One global_load_lds_dwordx4 moves 16
-// rows: four lanes cover the 64 contiguous bytes of a row.  The four 16-byte chunks of a row
-// are stored at position chunk ^ ((row / 4) % 4), which makes a fragment read (16 lanes = 16
-// consecutive rows, one chunk each) touch 16 different 16-byte bank groups.  Behind the ring:
+// LDS: two rings of 16 KB buffers, one for the routed rows and one for the weight rows.  A
+// buffer holds 64 contraction bytes -- one MFMA step, "slot" below -- of 256 rows, row-major.
+// One buffer_load_dwordx4 ... lds moves 16 rows: four lanes cover the 64 contiguous bytes of a
+// row.  The four 16-byte chunks of a row are stored at position chunk ^ ((row / 4) % 4), which
+// makes a fragment read (16 lanes = 16 consecutive rows, one chunk each) touch 16 different
+// 16-byte bank groups.  The weight ring has `depth` buffers (a link-time handle) and takes
+// one slot per step.  The routed-row ring has depth + 1 buffers and takes two slots -- the
+// two halves of one 128-byte line per row -- every second step, the two loads of a row back
+// to back: issued like that the pair costs the memory system what one full-line request
+// costs, issued a step apart it costs about a fifth more time (measured).  Behind the rings:
 // four 1 KB buffers of weight block scales (stored slot-major in HBM, one dword = 128
 // contraction bytes per row, so a tile's share is one contiguous load every second slot) and
 // two 4 KB buffers of routed-row scales (row-major in HBM because rows are gathered; 16 bytes
@@ -21,10 +26,9 @@
 //
 // Schedule: one wave per SIMD, 128 x 128 outputs per wave in 256 accumulator registers.
 // While the 16 MFMAs of slot j run, the wave reads the operands of slot j+1 from LDS into a
-// second register set and the loads of slot j+depth are in flight, so neither the LDS latency
-// nor the L2 latency sits between two MFMAs.  One s_barrier per slot; it only waits for what
-// was issued a full slot earlier.  The depth is a link-time handle; the ring offset inside
-// the workgroup's dynamic LDS is another.
+// second register set and the loads of the following slots are in flight, so neither the LDS
+// latency nor the L2 latency sits between two MFMAs.  One s_barrier per slot; it only waits
+// for what was issued `depth` - 1 steps earlier.
 #include <pipelink/stage.hpp>
 #ifndef PIPELINK_EMIT
 #include <type_traits>
@@ -41,7 +45,8 @@ using namespace mok;
 constexpr int WAVES = THREADS / 64;
 constexpr int X_GROUPS = TILE_X / 16 / WAVES;  // 16-row load groups per wave (4)
 constexpr int W_GROUPS = TILE_W / 16 / WAVES;  // (4)
-constexpr int TILE_LOADS = X_GROUPS + W_GROUPS;  // loads every wave issues for every slot, after the slot's scale loads
+constexpr int X_LOADS = 2 * X_GROUPS;          // loads of one routed-row pair issue (even steps)
+constexpr int W_LOADS = W_GROUPS;              // loads of one weight slot issue (every step)
 
 // Loads are buffer loads: a 128-bit resource (base address and byte extent, in scalar
 // registers), a 32-bit lane offset that is fixed for the tile, and the contraction offset as
@@ -71,31 +76,49 @@ struct Loader {
   uint32_t xscsrc;                // this thread's routed row in the scale matrix
   uint32_t xsrc[X_GROUPS];        // this lane's 16 bytes of its row in each group, at k = 0
   uint32_t wsrc[W_GROUPS];
-  int xdst, wdst;                 // slot-relative LDS byte offsets of the wave's first group
+  int dst;                        // buffer-relative LDS byte offset of the wave's first group (both rings)
+};
+
+// LDS areas of one workgroup
+struct Rings {
+  unsigned char* x;       // DEPTH + 1 buffers
+  unsigned char* w;       // DEPTH buffers
+  unsigned char* wscale;  // 4 x 1 KB
+  unsigned char* xscale;  // 2 x 4 KB
 };
 
 __device__ __forceinline__ int swizzle(int row) { return (row >> 2) & 3; }
 
-// Issue slot j into ring buffer `buf`.  Scale loads go first so that they are older than the
-// slot's tile loads: waiting until at most TILE_LOADS * m loads are outstanding then covers
-// every load of all but the youngest m slots, whatever scale loads those carried.
-// J8 is j % 8 where the caller knows it at compile time, else -1.
+// Issue the weight rows of slot j into weight buffer `buf`, preceded by the scale loads that
+// go with slot j.  Scale loads go first so that they are older than tile loads of the same
+// step: the outstanding-load counts the waits use only count tile loads, which errs on the
+// side of waiting for more.  J8 is j % 8 where the caller knows it at compile time, else -1.
 template <int J8 = -1>
-__device__ __forceinline__ void issue_slot(const Loader& ld, unsigned char* ring, unsigned char* wscale,
-                                           unsigned char* xscale, int j, int buf) {
+__device__ __forceinline__ void issue_w(const Loader& ld, const Rings& r, int j, int buf) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t kbyte = (uint32_t)j * K_SLOT;
   const int j8 = J8 >= 0 ? J8 : (j & 7);
-  unsigned char* slot = ring + buf * SLOT_BYTES;
   // every eighth slot: 16 scale bytes of each routed row (this slot and the next seven)
-  if (j8 == 0) buf16_to_lds(ld.xsc, ld.xscsrc, kbyte >> 5, xscale + ((j >> 3) & 1) * (TILE_X * 16) + wave * 1024);
+  if (j8 == 0) buf16_to_lds(ld.xsc, ld.xscsrc, kbyte >> 5, r.xscale + ((j >> 3) & 1) * (TILE_X * 16) + wave * 1024);
   // every second slot: the tile's weight scales of this pair, one row per thread
   if ((j8 & 1) == 0)
-    buf4_to_lds(ld.wsc, ld.wscsrc, (uint32_t)(j >> 1) * ld.wsc_pair_pitch, wscale + (j8 >> 1) * (TILE_W * 4) + wave * 256);
+    buf4_to_lds(ld.wsc, ld.wscsrc, (uint32_t)(j >> 1) * ld.wsc_pair_pitch, r.wscale + (j8 >> 1) * (TILE_W * 4) + wave * 256);
+  unsigned char* dst = r.w + buf * BUF_BYTES + ld.dst;
 #pragma unroll
-  for (int i = 0; i < X_GROUPS; ++i) buf16_to_lds(ld.x, ld.xsrc[i], kbyte, slot + ld.xdst + i * 1024);
+  for (int i = 0; i < W_GROUPS; ++i) buf16_to_lds(ld.w, ld.wsrc[i], kbyte, dst + i * 1024);
+}
+
+// Issue the routed rows of slots j and j+1 (j even: the two halves of a 128-byte line) into
+// routed-row buffers buf0 and buf1, the two loads of a row group back to back.
+__device__ __forceinline__ void issue_x_pair(const Loader& ld, const Rings& r, int j, int buf0, int buf1) {
+  const uint32_t kbyte = (uint32_t)j * K_SLOT;
+  unsigned char* dst0 = r.x + buf0 * BUF_BYTES + ld.dst;
+  unsigned char* dst1 = r.x + buf1 * BUF_BYTES + ld.dst;
 #pragma unroll
-  for (int i = 0; i < W_GROUPS; ++i) buf16_to_lds(ld.w, ld.wsrc[i], kbyte, slot + ld.wdst + i * 1024);
+  for (int i = 0; i < X_GROUPS; ++i) {
+    buf16_to_lds(ld.x, ld.xsrc[i], kbyte, dst0 + i * 1024);
+    buf16_to_lds(ld.x, ld.xsrc[i], kbyte + K_SLOT, dst1 + i * 1024);
+  }
 }
 
 // MFMA 32x32x64 f8f6f4 operand of lane (row = lane % 32, half = lane / 32): registers 0-3
@@ -132,12 +155,25 @@ struct Operands {
   v8i x[XFRAGS], w[WFRAGS];
 };
 
-__device__ __forceinline__ void read_operands(Operands& o, const unsigned char* slot, const int (&xoff)[XFRAGS],
-                                              const int (&woff)[WFRAGS]) {
+__device__ __forceinline__ void read_operands(Operands& o, const unsigned char* xbuf, const unsigned char* wbuf,
+                                              const int (&xoff)[XFRAGS], const int (&woff)[WFRAGS]) {
 #pragma unroll
-  for (int b = 0; b < XFRAGS; ++b) o.x[b] = read_frag(slot, xoff[b]);
+  for (int b = 0; b < XFRAGS; ++b) o.x[b] = read_frag(xbuf, xoff[b]);
 #pragma unroll
-  for (int a = 0; a < WFRAGS; ++a) o.w[a] = read_frag(slot, woff[a]);
+  for (int a = 0; a < WFRAGS; ++a) o.w[a] = read_frag(wbuf, woff[a]);
+}
+
+// s_waitcnt needs an immediate: the few counts the last steps of a tile can ask for
+__device__ __forceinline__ void wait_loads_and_reads_dyn(int n) {
+  switch (n) {
+    case 0: wait_loads_and_reads<0>(); break;
+    case 4: wait_loads_and_reads<4>(); break;
+    case 8: wait_loads_and_reads<8>(); break;
+    case 12: wait_loads_and_reads<12>(); break;
+    case 16: wait_loads_and_reads<16>(); break;
+    case 20: wait_loads_and_reads<20>(); break;
+    default: wait_loads_and_reads<0>(); break;  // waiting for everything is always right
+  }
 }
 
 // Block scales of the 128-byte pair that starts at slot j (j even): one dword per row; lanes
@@ -180,9 +216,12 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   const int expert = __builtin_amdgcn_readfirstlane(t.expert);
   const MokMxView& act = gate_up ? g.x : g.hidden;
   const int n = act.k / K_SLOT;  // the host rejects a contraction length that is not a multiple of 64
-  unsigned char* ring = pipelink_smem + pipelink_mok_gemm_arena();
-  unsigned char* wscale = ring + DEPTH * SLOT_BYTES;
-  unsigned char* xscale = wscale + WSCALE_BYTES;
+  constexpr int XDEPTH = DEPTH + 1;
+  Rings r;
+  r.x = pipelink_smem + pipelink_mok_gemm_arena();
+  r.w = r.x + XDEPTH * BUF_BYTES;
+  r.wscale = r.w + DEPTH * BUF_BYTES;
+  r.xscale = r.wscale + WSCALE_BYTES;
 
   // ---- loader addresses (fixed for the tile) ---------------------------------------
   // lane -> (row lane/4 of a 16-row group, LDS position lane%4); it fetches the chunk that
@@ -201,7 +240,8 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       ld.xsrc[i] = (uint32_t)src * (uint32_t)act.ld_q + chunk;
     }
     ld.x = make_rsrc(act.q, (uint32_t)act.rows * (uint32_t)act.ld_q);
-    ld.xdst = wave * X_GROUPS * 1024;
+    ld.dst = wave * X_GROUPS * 1024;
+    static_assert(X_GROUPS == W_GROUPS, "one wave offset serves both rings");
     const MokMxView& wv = gate_up ? (wave < WAVES / 2 ? g.w_gate : g.w_up) : g.w_down;
 #pragma unroll
     for (int i = 0; i < W_GROUPS; ++i) {
@@ -211,7 +251,6 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       ld.wsrc[i] = (uint32_t)col * (uint32_t)wv.ld_q + chunk;
     }
     ld.w = make_rsrc(wv.q + (int64_t)expert * wv.expert_pitch_q, (uint32_t)wv.rows * (uint32_t)wv.ld_q);
-    ld.wdst = SLOT_X_BYTES + wave * W_GROUPS * 1024;
     // routed-row scales: thread tid fetches row tid's 16-byte piece
     {
       int row = t.row_begin + tid;
@@ -244,7 +283,7 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
 #pragma unroll
   for (int a = 0; a < WFRAGS; ++a) {
     const int wl = wrow0(wave, a) + r32;
-    woff[a] = SLOT_X_BYTES + wl * K_SLOT + 16 * (half ^ swizzle(wl));
+    woff[a] = wl * K_SLOT + 16 * (half ^ swizzle(wl));
     wscoff[a] = wl * 4;
   }
 
@@ -255,30 +294,54 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc.v[a][b][r] = 0.0f;
 
-  // ---- prologue: fill the ring, fetch slot 0's operands --------------------------------
+  // Loads a step issues, in this order: [scale loads] [routed-row pair, even steps: X_LOADS]
+  // [weight slot: W_LOADS].  Step t needs slot t+1 in LDS.  Its weight rows were issued in step
+  // t+1-DEPTH; its routed rows in the even step t-DEPTH or t+1-DEPTH, in front of that step's
+  // weight rows.  So everything issued in steps t+2-DEPTH .. t-1 may still be outstanding.
+  auto issued_in = [&](int u) {  // tile loads step u issued (u < 0: the prologue plays steps -DEPTH .. -1)
+    const int s = u + DEPTH;     // slot whose weight rows step u issues
+    return (s < n ? W_LOADS : 0) + ((u & 1) == 0 && s < n ? X_LOADS : 0);
+  };
+  constexpr int STEADY = (DEPTH - 2) * W_LOADS + (DEPTH - 2) / 2 * X_LOADS;  // DEPTH is even
+  static_assert(DEPTH % 2 == 0, "routed-row pairs are issued on even steps");
+
+  // ---- prologue: steps -DEPTH .. -1 of the schedule, then slot 0's operands --------------
 #pragma unroll
-  for (int s = 0; s < DEPTH; ++s)
-    if (s < n) issue_slot(ld, ring, wscale, xscale, s, s);
-  if (n >= DEPTH)
-    wait_loads_and_reads<TILE_LOADS * (DEPTH - 1)>();
-  else
-    wait_loads_and_reads<0>();
+  for (int u = -DEPTH; u < 0; ++u) {
+    const int s = u + DEPTH;
+    if (s < n) {
+      if ((s & 1) == 0) issue_x_pair(ld, r, s, s, s + 1);
+      issue_w(ld, r, s, s);
+    }
+  }
+  {  // slot 0: younger loads are those of prologue steps 1-DEPTH .. -1
+    int younger = 0;
+#pragma unroll
+    for (int u = 1 - DEPTH; u < 0; ++u) younger += issued_in(u);
+    wait_loads_and_reads_dyn(younger);
+  }
   wg_barrier();
   Operands even, odd;
   int sx[XFRAGS], sw[WFRAGS], sxn[XFRAGS], swn[WFRAGS];
-  read_operands(even, ring, xoff, woff);
-  read_scales(sx, sw, wscale, xscale, 0, xscoff, wscoff, half);
+  read_operands(even, r.x, r.w, xoff, woff);
+  read_scales(sx, sw, r.wscale, r.xscale, 0, xscoff, wscoff, half);
 
   // Step j multiplies slot j (already in registers) while it fetches slot j+1's operands from
   // LDS; the barrier in front says slot j+1 has landed for every wave and every wave holds
-  // slot j in registers, so slot j's buffer takes the loads of slot j+DEPTH.
+  // slot j in registers, so slot j's buffers are free.
   //
   // Steady state: groups of eight steps, fully unrolled, as long as every step of the group
-  // still has a slot to issue.  Ring buffer, scale buffer, scale byte and the slots that carry
-  // scale loads are compile-time constants there, so the group is one basic block and the
-  // MFMAs stay where they are written, between the LDS reads they overlap with.
-  static_assert(8 % DEPTH == 0, "a group of eight slots must start at ring buffer 0");
+  // still has slots to issue.  Weight buffer, scale buffer, scale byte and the slots that carry
+  // scale loads are compile-time constants there (the routed-row buffer, modulo DEPTH + 1, is
+  // not), so the group is one basic block and the MFMAs stay where they are written, between
+  // the LDS reads they overlap with.
+  static_assert(8 % DEPTH == 0, "a group of eight slots must start at weight buffer 0");
   int j = 0;
+  int xb = 0;  // routed-row buffer of slot j
+  auto xnext = [](int b, int by) {  // (b + by) mod XDEPTH for 0 <= b < XDEPTH, 0 <= by <= XDEPTH
+    const int c = b + by;
+    return c >= XDEPTH ? c - XDEPTH : c;
+  };
   for (; j + 8 + DEPTH <= n; j += 8) {
     auto step = [&](auto S_) {
       constexpr int S = decltype(S_)::value;
@@ -286,20 +349,24 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       Operands& cur = ODD ? odd : even;
       Operands& next = ODD ? even : odd;
       __builtin_amdgcn_sched_barrier(0);  // nothing of the previous step sinks below, nothing of this one rises above
-      wait_loads_and_reads<TILE_LOADS * (DEPTH - 2)>();  // loads younger than slot j+S+1's: DEPTH-2 slots
+      wait_loads_and_reads<STEADY>();
       wg_barrier();
-      issue_slot<(S + DEPTH) & 7>(ld, ring, wscale, xscale, j + S + DEPTH, S % DEPTH);
-      read_operands(next, ring + ((S + 1) % DEPTH) * SLOT_BYTES, xoff, woff);
-      if (ODD) read_scales<(S + 1) & 7>(sxn, swn, wscale, xscale, j + S + 1, xscoff, wscoff, half);
+      // slot j+S's buffers are free; so is the routed-row buffer before it (freed a step ago)
+      const int xprev = xnext(xb, XDEPTH - 1);
+      if (!ODD) issue_x_pair(ld, r, j + S + DEPTH, xprev, xb);
+      issue_w<(S + DEPTH) & 7>(ld, r, j + S + DEPTH, S % DEPTH);
+      xb = xnext(xb, 1);
+      read_operands(next, r.x + xb * BUF_BYTES, r.w + ((S + 1) % DEPTH) * BUF_BYTES, xoff, woff);
+      if (ODD) read_scales<(S + 1) & 7>(sxn, swn, r.wscale, r.xscale, j + S + 1, xscoff, wscoff, half);
       mma_step<ODD>(cur, sx, sw, acc);
       // issue order inside the step: an MFMA first (the pipe must not drain behind the
-      // barrier), the global loads spread over the first eight MFMAs, the LDS reads over the rest
+      // barrier), the global loads spread over the first MFMAs, the LDS reads over the rest
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
       __builtin_amdgcn_sched_group_barrier(0x010, 3, 0);  // VMEM: the scale loads and the first tile load
 #pragma unroll
       for (int i = 1; i < 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);  // VMEM
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x010, ODD ? 1 : 2, 0);  // VMEM
       }
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -325,25 +392,28 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   }
 
   // Remaining slots (fewer than 8 + DEPTH), same steps with run-time slot numbers.  The MFMA
-  // chain is straight-line code: past the last slot `advance` still runs (it reads a buffer
+  // chain is straight-line code: past the last slot `advance` still runs (it reads buffers
   // nobody uses), which keeps control flow out of the accumulator's live range.
-  int buf = 0;  // ring buffer of slot j (j is a multiple of 8 here)
-  auto advance = [&](int jj, Operands& next) {
-    // loads younger than slot jj+1's: slots jj+2 .. jj+DEPTH-1, if all of those exist
-    if (jj + DEPTH <= n)
-      wait_loads_and_reads<TILE_LOADS * (DEPTH - 2)>();
-    else
-      wait_loads_and_reads<0>();
+  int wb = 0;  // weight buffer of slot j (j is a multiple of 8 here)
+  auto advance = [&](int t_, Operands& next) {
+    int younger = 0;
+#pragma unroll
+    for (int u = 2 - DEPTH; u < 0; ++u) younger += issued_in(t_ + u);
+    wait_loads_and_reads_dyn(younger);
     wg_barrier();
-    if (jj + DEPTH < n) issue_slot(ld, ring, wscale, xscale, jj + DEPTH, buf);
-    buf = buf + 1 == DEPTH ? 0 : buf + 1;
-    read_operands(next, ring + buf * SLOT_BYTES, xoff, woff);
+    if (t_ + DEPTH < n) {
+      if ((t_ & 1) == 0) issue_x_pair(ld, r, t_ + DEPTH, xnext(xb, XDEPTH - 1), xb);
+      issue_w(ld, r, t_ + DEPTH, wb);
+    }
+    xb = xnext(xb, 1);
+    wb = wb + 1 == DEPTH ? 0 : wb + 1;
+    read_operands(next, r.x + xb * BUF_BYTES, r.w + wb * BUF_BYTES, xoff, woff);
   };
   for (; j + 1 < n; j += 2) {
     advance(j, odd);
     mma_step<false>(even, sx, sw, acc);
     advance(j + 1, even);
-    read_scales(sxn, swn, wscale, xscale, j + 2, xscoff, wscoff, half);
+    read_scales(sxn, swn, r.wscale, r.xscale, j + 2, xscoff, wscoff, half);
     mma_step<true>(odd, sx, sw, acc);
 #pragma unroll
     for (int b = 0; b < XFRAGS; ++b) sx[b] = sxn[b];
@@ -369,7 +439,7 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 
 template <int DEPTH>
 __device__ __forceinline__ void store_down(const MokGemmResidue& g, const MokGemmTask& t, const AccFrag& acc) {
-  constexpr int RING_BYTES = DEPTH * SLOT_BYTES + WSCALE_BYTES + XSCALE_BYTES;
+  constexpr int RING_BYTES = (2 * DEPTH + 1) * BUF_BYTES + WSCALE_BYTES + XSCALE_BYTES;
   constexpr int PASSES = TILE_X * Y_PITCH <= RING_BYTES ? 1 : 2;
   constexpr int ROWS = TILE_X / PASSES;  // rows staged per pass
   static_assert(ROWS * Y_PITCH <= RING_BYTES, "half a tile must fit the ring");
@@ -447,9 +517,9 @@ PL_EXPORT(mok_gemm_fwd, mok_gemm_fwd,
           "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc);");
 PL_SERVE(gemm_init, "mok_gemm_init");
 PL_SERVE(gemm_fwd, "mok_gemm_fwd");
-// ring of `depth` slots: 256 x 64 B of routed rows, 256 x 64 B of weight rows
-// + 12 KB behind the ring: four 1 KB buffers of weight scales, two 4 KB buffers of routed-row scales
-PL_CLAIM_RING("pipelink_mok_gemm_arena", "smem", 12288, "pipelink_mok_gemm_depth", 32768, 1024, "phase:instr_gemm");
+// per unit of depth one 16 KB weight buffer and one 16 KB routed-row buffer; fixed: the extra routed-row
+// buffer, four 1 KB buffers of weight scales, two 4 KB buffers of routed-row scales
+PL_CLAIM_RING("pipelink_mok_gemm_arena", "smem", 16384 + 12288, "pipelink_mok_gemm_depth", 32768, 1024, "phase:instr_gemm");
 PL_USES("pipelink_mok_gemm_depth");
 PL_USES("pipelink_mok_gemm_arena");
 PL_FACT("mok.gemm.TILE_X", 256);

@@ -26,9 +26,7 @@ constexpr int K_PAIR = 128;     // contraction bytes one dword of four e8m0 bloc
 constexpr int WFRAGS = 4;       // 32-row weight fragments per wave
 constexpr int XFRAGS = 4;       // 32-row activation fragments per wave
 constexpr int THREADS = 256;
-constexpr int SLOT_X_BYTES = TILE_X * K_SLOT;
-constexpr int SLOT_W_BYTES = TILE_W * K_SLOT;
-constexpr int SLOT_BYTES = SLOT_X_BYTES + SLOT_W_BYTES;  // 32768
+constexpr int BUF_BYTES = TILE_X * K_SLOT;                // one ring buffer: 256 rows x 64 bytes (TILE_W == TILE_X)
 constexpr int WSCALE_BYTES = 4 * TILE_W * 4;             // four buffers of one dword (4 block scales) per weight row
 constexpr int XSCALE_BYTES = 2 * TILE_X * 16;            // two buffers of 16 scale bytes (8 slots) per routed row
 
