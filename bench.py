@@ -5,7 +5,7 @@ MXFP8 requant -> down grouped GEMM -> bf16) on one MI355X.
 One step = one forward over the whole batch: T=8192 tokens, d_model=d_ff=2880, 32 experts,
 top-4 routing (32768 routed rows), inputs already resident in HBM.  Prints ONE JSON line:
 metric = MXFP8 grouped-GEMM TFLOP/s on the algorithmic (unpadded) flop count
-2*R*H*I*3 = 1.6307e12 per forward, plus
+2*R*H*I*3 = 1.6307e12 per forward (weights in the layouts the kernel streams: K-tiled codes, slot-major scales), plus
   roofline      -- the gate/up pass (the dominant kernel) timed with HIP events on its launch
                    stream, against the 5.0 PFLOP/s dense FP8 MFMA peak;
   cpu_baseline  -- the CPU oracle (torch fp32 dequant-then-matmul) timed on the host cores on
@@ -39,7 +39,8 @@ def make_inputs(dev, seed=0):
     time); quantised on the device (bit-exact with the host rule) into 128-byte-pitched rows."""
     import torch
     from pipelink_amd.host import mok_inputs
-    from pipelink_amd.host.mok import code_pitch, mxfp8_quantize_device, weight_scales_to_slot_major
+    from pipelink_amd.host.mok import (code_pitch, mxfp8_quantize_device, weight_codes_to_k64_tiled,
+                                       weight_scales_to_slot_major)
 
     g = torch.Generator().manual_seed(seed)
     logits = torch.randn(T, E, generator=g)
@@ -51,17 +52,20 @@ def make_inputs(dev, seed=0):
         qs, scs = [], []
         for _ in range(E):
             w = torch.randn(n, k, generator=g) * 0.02
-            q, sc = mxfp8_quantize_device(w.to(dev), code_pitch(k))
+            q, sc = mxfp8_quantize_device(w.to(dev), k)
             qs.append(q)
             scs.append(sc)
-        return torch.stack(qs), torch.stack(scs), weight_scales_to_slot_major(torch.stack(scs), k)
+        q, sc = torch.stack(qs), torch.stack(scs)
+        # (K-tiled codes, row-major scales, slot-major scales, row-major codes)
+        return weight_codes_to_k64_tiled(q, k), sc, weight_scales_to_slot_major(sc, k), q
 
     wg = weights(I, H)
     wu = weights(I, H)
     wd = weights(H, I)
     dev_args = dict(tokens_per_expert=counts.to(dev), row_token=row_token.to(dev), x_q=x_q, x_sc=x_sc, w_gate_q=wg[0],
                     w_gate_sc=wg[2], w_up_q=wu[0], w_up_sc=wu[2], w_down_q=wd[0], w_down_sc=wd[2])
-    row_major = dict(w_gate_sc=wg[1], w_up_sc=wu[1], w_down_sc=wd[1])  # what the CPU oracle reads
+    # what the CPU oracle reads: row-major codes and scales
+    row_major = dict(w_gate_sc=wg[1], w_up_sc=wu[1], w_down_sc=wd[1], w_gate_q=wg[3], w_up_q=wu[3], w_down_q=wd[3])
     return dev_args, row_major
 
 

@@ -10,14 +10,16 @@
  * and the down pass on the caller's stream.  All tensor arguments are device addresses
  * owned by the caller; nothing is allocated per call.
  *
- * Operand layouts (all row-major; a code row may be padded to a pitch ld_q >= K, a multiple
- * of 16 -- a pitch that is a multiple of 128 makes every ring-slot row one aligned cache
- * line, which is what the loader is fastest on):
- *   x_q [T,H] e4m3, x_sc [T,ld_sc_h] e8m0 (one byte per 32 elements of H; ld_sc_h % 16 == 0)
- *   w_gate_q / w_up_q [E,I,H], w_down_q [E,H,I]; weight scales are SLOT-MAJOR:
- *   [E, ceil(K/128), N, 4] (the 4 scale bytes of one 128-element K-slot of one row are a dword,
- *   and one slot's dwords of consecutive rows are contiguous) -- convert a row-major scale
- *   matrix once, when the weights are loaded, with plk_mxfp8_scales_to_slot_major
+ * Operand layouts.  Activations are row-major; a code row may be padded to a pitch ld_q >= K,
+ * a multiple of 16 -- a pitch that is a multiple of 128 makes every 128-byte piece of a row
+ * one aligned cache line, which is what the loader is fastest on:
+ *   x_q [T,ld_q_h] e4m3, x_sc [T,ld_sc_h] e8m0 (one byte per 32 elements of H; ld_sc_h % 16 == 0)
+ * Weights are stored the way the GEMM streams them; convert once, when the weights are loaded:
+ *   w_gate_q / w_up_q (N = I, K = H), w_down_q (N = H, K = I): K-TILED codes [E, K/64, N, 64]
+ *   (64 contraction bytes of consecutive rows are contiguous) -- plk_mxfp8_codes_to_k64_tiled
+ *   weight scales SLOT-MAJOR [E, ceil(K/128), N, 4] (the 4 scale bytes of 128 contraction
+ *   elements of one row are a dword, and one slot's dwords of consecutive rows are
+ *   contiguous) -- plk_mxfp8_scales_to_slot_major
  *   tokens_per_expert [E] i32, row_token [R] i32 (routed row -> token; 0 = rows are tokens)
  *   hidden_q [R,I] e4m3 + hidden_sc [R,ld_sc_i] (written by pass 1, read by pass 2)
  *   y [R,H] bf16 */
@@ -51,8 +53,8 @@ typedef struct plk_mok_problem {
   int32_t routed_rows;   /* R = sum(tokens_per_expert) */
   int32_t ld_sc_h;       /* scale row pitch for K = H operands */
   int32_t ld_sc_i;       /* scale row pitch for K = I operands */
-  int32_t ld_q_h;        /* code row pitch in bytes for K = H operands (x, w_gate, w_up); 0 = H */
-  int32_t ld_q_i;        /* code row pitch in bytes for K = I operands (hidden, w_down); 0 = I */
+  int32_t ld_q_h;        /* code row pitch in bytes of x; 0 = H */
+  int32_t ld_q_i;        /* code row pitch in bytes of hidden; 0 = I */
   float swiglu_limit;
   int32_t reserved;
   uint64_t x_q, x_sc, row_token, tokens_per_expert;
@@ -79,6 +81,10 @@ int plk_mxfp8_quantize(uint64_t src, int src_is_bf16, int64_t rows, int32_t k, u
  * For a weight tensor [E, N, K] call it once per expert (or once with rows = E*N when the
  * caller wants one slot-major block per expert, use rows = N and offset the pointers). */
 int plk_mxfp8_scales_to_slot_major(uint64_t src, int64_t rows, int32_t k, int32_t ld_sc, uint64_t dst, void* stream);
+
+/* Row-major e4m3 codes src [rows, ld_q] -> K-tiled dst [k/64, rows, 64] (k % 64 == 0, ld_q % 16 == 0,
+ * 16-byte aligned addresses).  For a weight tensor [E, N, K] call it once per expert with rows = N. */
+int plk_mxfp8_codes_to_k64_tiled(uint64_t src, int64_t rows, int32_t k, int64_t ld_q, uint64_t dst, void* stream);
 
 #ifdef __cplusplus
 }

@@ -48,8 +48,7 @@ static int check_problem(const plk_mok_problem* p) {
     // the kernel addresses one operand with 32-bit byte offsets from its base
     const int64_t ldh = p->ld_q_h ? p->ld_q_h : p->hidden, ldi = p->ld_q_i ? p->ld_q_i : p->intermediate;
     const int64_t lim = (int64_t)1 << 32;
-    if (p->num_tokens * ldh >= lim || p->routed_rows * ldi >= lim || (int64_t)p->intermediate * ldh >= lim ||
-        (int64_t)p->hidden * ldi >= lim)
+    if (p->num_tokens * ldh >= lim || p->routed_rows * ldi >= lim || (int64_t)p->intermediate * p->hidden >= lim)
       return plk_hip_set_error(PLK_E_CAPACITY, "plk_mok: an operand (rows x row pitch) must stay below 4 GiB");
   }
   if (p->routed_rows && (!p->x_q || !p->x_sc || !p->tokens_per_expert || !p->w_gate_q || !p->w_gate_sc ||
@@ -59,16 +58,17 @@ static int check_problem(const plk_mok_problem* p) {
   return PLK_OK;
 }
 
-// activations: row-major scales with pitch ld_sc; weights (per_expert): slot-major scales [slots, rows, 4]
+// activations: row-major codes with pitch ld_q, row-major scales with pitch ld_sc;
+// weights (per_expert): K-tiled codes [K/64, rows, 64], slot-major scales [K/128, rows, 4]
 static MokMxView view(uint64_t q, uint64_t sc, int64_t rows, int k, int ld_q, int ld_sc, bool per_expert) {
   MokMxView v{};
   v.q = (const uint8_t*)(uintptr_t)q;
   v.sc = (const uint8_t*)(uintptr_t)sc;
   v.rows = (int32_t)rows;
   v.k = k;
-  v.ld_q = ld_q;
+  v.ld_q = per_expert ? 64 : ld_q;
   v.ld_sc = ld_sc;
-  v.expert_pitch_q = per_expert ? rows * (int64_t)ld_q : 0;
+  v.expert_pitch_q = per_expert ? rows * (int64_t)k : 0;
   v.expert_pitch_sc = per_expert ? (int64_t)((k + 127) / 128) * rows * 4 : 0;
   return v;
 }
@@ -247,6 +247,32 @@ extern "C" int plk_mxfp8_quantize(uint64_t src, int src_is_bf16, int64_t rows, i
   else
     mxfp8_quantize_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>(
         (const void*)(uintptr_t)src, rows, k, (uint8_t*)(uintptr_t)dst_q, ld_q, (uint8_t*)(uintptr_t)dst_sc, ld_sc);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return plk_hip_set_error(PLK_E_RESOURCE, hipGetErrorString(e));
+  return PLK_OK;
+}
+
+// ---- weight code layout conversion: row-major [rows, ld_q] -> K-tiled [K/64, rows, 64] ------
+__global__ void __launch_bounds__(256) codes_to_k64_tiled_kernel(const uint8_t* __restrict__ src, int64_t rows, int ktiles,
+                                                                  int64_t ld_q, uint8_t* __restrict__ dst) {
+  const int64_t total = rows * (int64_t)ktiles * 4;  // 16-byte pieces
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int c = (int)(i & 3);
+    const int64_t rt = i >> 2, kt = rt / rows, r = rt - kt * rows;
+    const uint4 v = *reinterpret_cast<const uint4*>(src + r * ld_q + kt * 64 + c * 16);
+    *reinterpret_cast<uint4*>(dst + i * 16) = v;
+  }
+}
+
+extern "C" int plk_mxfp8_codes_to_k64_tiled(uint64_t src, int64_t rows, int32_t k, int64_t ld_q, uint64_t dst, void* stream) {
+  if (rows < 0 || k <= 0 || k % 64 || ld_q < k || ld_q % 16 || (src & 15) || (dst & 15))
+    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mxfp8_codes_to_k64_tiled: k must be a positive multiple of 64, ld_q a multiple of 16 not below k, addresses 16-byte aligned");
+  if (rows == 0) return PLK_OK;
+  if (!src || !dst) return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mxfp8_codes_to_k64_tiled: null device address");
+  int64_t grid = (rows * (k / 64) * 4 + 255) / 256;
+  if (grid > 65536) grid = 65536;
+  codes_to_k64_tiled_kernel<<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>(
+      (const uint8_t*)(uintptr_t)src, rows, k / 64, ld_q, (uint8_t*)(uintptr_t)dst);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return plk_hip_set_error(PLK_E_RESOURCE, hipGetErrorString(e));
   return PLK_OK;

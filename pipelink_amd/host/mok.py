@@ -41,6 +41,21 @@ def weight_scales_to_slot_major(sc: torch.Tensor, k: int) -> torch.Tensor:
     return out
 
 
+def weight_codes_to_k64_tiled(q: torch.Tensor, k: int) -> torch.Tensor:
+    """Row-major weight codes [E, N, ld] (ld >= k) -> the K-tiled layout the GEMM streams, [E, k/64, N, 64]."""
+    if not q.is_cuda or not q.is_contiguous() or q.dim() != 3 or q.dtype != torch.uint8:
+        raise PlkError(3, "codes must be a contiguous 3-D uint8 device tensor")
+    e, n, ld = q.shape
+    if k % 64 or ld < k:
+        raise PlkError(3, "k must be a multiple of 64 and not exceed the row pitch")
+    out = torch.empty((e, k // 64, n, 64), dtype=torch.uint8, device=q.device)
+    lib = load_library()
+    stream = c_void_p(torch.cuda.current_stream().cuda_stream)
+    for i in range(e):
+        check(lib, lib.plk_mxfp8_codes_to_k64_tiled(q[i].data_ptr(), n, k, ld, out[i].data_ptr(), stream))
+    return out
+
+
 def link_info_from_json(link: dict) -> MokLinkInfo:
     """Translate a ``link.json`` (pipec link output) into the C record the session wants."""
     entries = {e["stage_id"]: e for e in link["params"]["entries"]}
@@ -84,13 +99,17 @@ class MoKSession:
                             w_down_sc=w_down_sc, hidden_q=hidden_q, hidden_sc=hidden_sc, y=y).items():
             if not t.is_cuda or not t.is_contiguous():
                 raise PlkError(3, f"{name} must be a contiguous device tensor")
-        # code tensors may carry a padded last dimension (row pitch); the logical K comes from y / w_down
+        # activation code tensors may carry a padded last dimension (row pitch); the logical sizes come from
+        # y [R, H] and the K-tiled weights [E, K/64, N, 64]
         t_rows, ldh = x_q.shape
         r, h = y.shape
-        e, i, ldh2 = w_gate_q.shape
+        if w_gate_q.dim() != 4 or w_gate_q.shape[3] != 64:
+            raise PlkError(3, "weight codes must be K-tiled [E, K/64, N, 64] (see weight_codes_to_k64_tiled)")
+        e, _, i, _ = w_gate_q.shape
         ldi_q = hidden_q.shape[1]
-        if ldh2 != ldh or tuple(w_up_q.shape) != (e, i, ldh) or tuple(w_down_q.shape) != (e, h, ldi_q):
-            raise PlkError(3, "weight shapes disagree with x / hidden")
+        if h % 64 or i % 64 or tuple(w_gate_q.shape) != (e, h // 64, i, 64) or tuple(w_up_q.shape) != (e, h // 64, i, 64) or \
+                tuple(w_down_q.shape) != (e, i // 64, h, 64):
+            raise PlkError(3, "weight shapes disagree with y / each other")
         if hidden_q.shape[0] != r or y.dtype != torch.bfloat16 or ldh < h or ldi_q < i:
             raise PlkError(3, "hidden_q / y shapes disagree")
         ldsh, ldsi = scale_pitch(h), scale_pitch(i)

@@ -15,7 +15,8 @@
 // row.  The four 16-byte chunks of a row are stored at position chunk ^ ((row / 4) % 4), which
 // makes a fragment read (16 lanes = 16 consecutive rows, one chunk each) touch 16 different
 // 16-byte bank groups.  The weight ring has `depth` buffers (a link-time handle) and takes
-// one slot per step.  The routed-row ring has depth + 1 buffers and takes two slots -- the
+// one slot per step; weight codes are stored K-tiled in HBM ([K/64][rows][64 bytes]), so the
+// 16 rows of a load are 1 KB of contiguous memory.  The routed-row ring has depth + 1 buffers and takes two slots -- the
 // two halves of one 128-byte line per row -- every second step, the two loads of a row back
 // to back: issued like that the pair costs the memory system what one full-line request
 // costs, issued a step apart it costs about a fifth more time (measured).  Behind the rings:
@@ -72,6 +73,7 @@ struct Loader {
   rsrc_t xsc;                     // routed rows' scales, row-major
   rsrc_t wsc;                     // this expert's weight scales (gate or up or down, by wave), slot-major
   uint32_t wsc_pair_pitch;        // bytes between two 128-byte pairs of the weight scales
+  uint32_t w_slot_pitch;          // bytes between two 64-byte slots of the weight codes (K-tiled: rows x 64)
   uint32_t wscsrc;                // this thread's weight row: its dword of block scales
   uint32_t xscsrc;                // this thread's routed row in the scale matrix
   uint32_t xsrc[X_GROUPS];        // this lane's 16 bytes of its row in each group, at k = 0
@@ -104,8 +106,9 @@ __device__ __forceinline__ void issue_w(const Loader& ld, const Rings& r, int j,
   if ((j8 & 1) == 0)
     buf4_to_lds(ld.wsc, ld.wscsrc, (uint32_t)(j >> 1) * ld.wsc_pair_pitch, r.wscale + (j8 >> 1) * (TILE_W * 4) + wave * 256);
   unsigned char* dst = r.w + buf * BUF_BYTES + ld.dst;
+  const uint32_t wslot = (uint32_t)j * ld.w_slot_pitch;
 #pragma unroll
-  for (int i = 0; i < W_GROUPS; ++i) buf16_to_lds(ld.w, ld.wsrc[i], kbyte, dst + i * 1024);
+  for (int i = 0; i < W_GROUPS; ++i) buf16_to_lds(ld.w, ld.wsrc[i], wslot, dst + i * 1024);
 }
 
 // Issue the routed rows of slots j and j+1 (j even: the two halves of a 128-byte line) into
@@ -248,9 +251,10 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       const int wl = (wave * W_GROUPS + i) * 16 + lrow;  // tile-local weight row
       int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
       col = col < wv.rows ? col : wv.rows - 1;
-      ld.wsrc[i] = (uint32_t)col * (uint32_t)wv.ld_q + chunk;
+      ld.wsrc[i] = (uint32_t)col * (uint32_t)K_SLOT + chunk;  // weights are K-tiled: [K/64][rows][64]
     }
-    ld.w = make_rsrc(wv.q + (int64_t)expert * wv.expert_pitch_q, (uint32_t)wv.rows * (uint32_t)wv.ld_q);
+    ld.w = make_rsrc(wv.q + (int64_t)expert * wv.expert_pitch_q, (uint32_t)wv.rows * (uint32_t)wv.k);
+    ld.w_slot_pitch = (uint32_t)wv.rows * (uint32_t)K_SLOT;
     // routed-row scales: thread tid fetches row tid's 16-byte piece
     {
       int row = t.row_begin + tid;

@@ -31,20 +31,20 @@ def cell():
 
 
 def _run(sess, inp, H, I, pitch_h=None, pitch_i=None, limit=7.0):
-    from pipelink_amd.host.mok import scale_pitch, weight_scales_to_slot_major
+    from pipelink_amd.host.mok import scale_pitch, weight_codes_to_k64_tiled, weight_scales_to_slot_major
 
     dev = torch.device("cuda:0")
     d = {k: v.to(dev) for k, v in inp.__dict__.items()}
     d["w_gate_sc"] = weight_scales_to_slot_major(d["w_gate_sc"], H)   # the layout the GEMM reads
     d["w_up_sc"] = weight_scales_to_slot_major(d["w_up_sc"], H)
     d["w_down_sc"] = weight_scales_to_slot_major(d["w_down_sc"], I)
-    if pitch_h:  # re-pitch the K = H operands
-        def pad(t, p):
-            out = torch.zeros(t.shape[:-1] + (p,), dtype=torch.uint8, device=dev)
-            out[..., :t.shape[-1]] = t
-            return out
-        d["x_q"], d["w_gate_q"], d["w_up_q"] = pad(d["x_q"], pitch_h), pad(d["w_gate_q"], pitch_h), pad(d["w_up_q"], pitch_h)
-        d["w_down_q"] = pad(d["w_down_q"], pitch_i)
+    if pitch_h:  # re-pitch the activation rows
+        out = torch.zeros((d["x_q"].shape[0], pitch_h), dtype=torch.uint8, device=dev)
+        out[:, :H] = d["x_q"]
+        d["x_q"] = out
+    d["w_gate_q"] = weight_codes_to_k64_tiled(d["w_gate_q"], H)       # the layout the GEMM streams
+    d["w_up_q"] = weight_codes_to_k64_tiled(d["w_up_q"], H)
+    d["w_down_q"] = weight_codes_to_k64_tiled(d["w_down_q"], I)
     rows = int(inp.tokens_per_expert.sum())
     hq = torch.full((rows, pitch_i or I), 0xFF, dtype=torch.uint8, device=dev)       # poison
     hsc = torch.full((rows, scale_pitch(I)), 0xFF, dtype=torch.uint8, device=dev)
