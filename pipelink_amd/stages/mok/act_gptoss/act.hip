@@ -59,7 +59,7 @@ __device__ __forceinline__ uint32_t pack_e4m3x4(float a, float b, float c, float
 
 template <bool CLAMPED>
 __device__ __forceinline__ void forward(const MokActResidue& p, const MokActTask& t, const AccFrag& acc) {
-  const int tid = threadIdx.x;
+  const int tid = fresh_tid();
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int half = lane >> 5;

@@ -18,8 +18,10 @@ extern "C" __device__ int pipelink_mok_fw_sched();  // byte offset of the schedu
 
 extern "C" __device__ void pipelink_call_gemm_init(const void* view);
 extern "C" __device__ void pipelink_call_act_init(const void* view);
+extern "C" __device__ void pipelink_call_gemm_prefetch(const void* view, const MokGemmTask*, mok::GemmCarry*);
 extern "C" __device__ void pipelink_call_gemm_fwd(const void* view, const MokGemmTask*, const MokCounters*, uint32_t*,
-                                                  mok::AccFrag*);
+                                                  mok::AccFrag*, const mok::GemmCarry*);
+extern "C" __device__ void pipelink_call_gemm_store(const void* view, const MokGemmTask*, const mok::AccFrag*);
 extern "C" __device__ void pipelink_call_act_fwd(const void* view, const MokActTask*, const MokCounters*, uint32_t*,
                                                  const mok::AccFrag*);
 
@@ -66,27 +68,49 @@ extern "C" __device__ void mok_framework_worker(const void* params, unsigned var
   const MokCounters counters{nullptr};
   uint32_t phase = 0;
 
-  for (int idx = xcd * chunk + blockIdx.x / NUM_XCD; idx < chunk_end; idx += per_xcd) {
+  const bool gate_up = g.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
+  auto decode = [&](int idx) {
     // expert of tile idx: last e with tile_begin[e] * nct <= idx
     int lo = 0, hi = ne;
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
       if (tile_begin[mid] * nct <= idx) lo = mid; else hi = mid;
     }
-    const int e = lo;
+    const int e = __builtin_amdgcn_readfirstlane(lo);
     const int mtiles = tile_begin[e + 1] - tile_begin[e];
     const int local = idx - tile_begin[e] * nct;
     const int nt = local / mtiles;
     const int mt = local - nt * mtiles;
-    const bool gate_up = g.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
     const int col_begin = nt * (gate_up ? mok::TILE_W / 2 : mok::TILE_W);
-    const MokGemmTask task{g.op, e, row_begin[e] + mt * mok::TILE_X, row_begin[e + 1], col_begin, idx, 0u};
+    // wave-uniform by construction; say so, so that the task lives in scalar registers
+    return MokGemmTask{g.op, e, __builtin_amdgcn_readfirstlane(row_begin[e] + mt * mok::TILE_X),
+                       __builtin_amdgcn_readfirstlane(row_begin[e + 1]), __builtin_amdgcn_readfirstlane(col_begin), idx, 0u};
+  };
+
+  // Software pipeline over this workgroup's tiles: the next tile's first loads are issued
+  // between a tile's mainloop and its epilogue, so they fly while the epilogue computes.
+  int idx = xcd * chunk + blockIdx.x / NUM_XCD;
+  if (idx >= chunk_end) return;
+  MokGemmTask task = decode(idx);
+  mok::GemmCarry carry;
+  pipelink_call_gemm_prefetch(&view, &task, &carry);
+  for (;;) {
+    const int next_idx = idx + per_xcd;
+    const bool has_next = next_idx < chunk_end;
+    MokGemmTask next = task;
+    if (has_next) next = decode(next_idx);
     mok::AccFrag acc;
-    pipelink_call_gemm_fwd(&view, &task, &counters, &phase, &acc);
+    pipelink_call_gemm_fwd(&view, &task, &counters, &phase, &acc, &carry);
+    if (has_next) pipelink_call_gemm_prefetch(&view, &next, &carry);
     if (gate_up) {
-      const MokActTask act{MOK_ACT_FWD_ROUTED, task.row_begin, task.row_end, col_begin, idx, 0u};
+      const MokActTask act{MOK_ACT_FWD_ROUTED, task.row_begin, task.row_end, task.col_begin, idx, 0u};
       pipelink_call_act_fwd(&view, &act, &counters, &phase, &acc);
+    } else {
+      pipelink_call_gemm_store(&view, &task, &acc);
     }
+    if (!has_next) break;
+    task = next;
+    idx = next_idx;
   }
 }
 #else  // PIPELINK_EMIT: host-evaluated annotations only
@@ -100,9 +124,13 @@ PL_TOPOLOGY(true, "static");
 PL_VARIANT(0, {});
 PL_CALL(gemm_init, "mok_gemm_init", "extern \"C\" __device__ void pipelink_call_gemm_init(const void* view);");
 PL_CALL(act_init, "mok_act_init", "extern \"C\" __device__ void pipelink_call_act_init(const void* view);");
+PL_CALL(gemm_prefetch, "mok_gemm_prefetch",
+        "extern \"C\" __device__ void pipelink_call_gemm_prefetch(const void* view, const MokGemmTask* task, mok::GemmCarry* carry);");
 PL_CALL(gemm_fwd, "mok_gemm_fwd",
         "extern \"C\" __device__ void pipelink_call_gemm_fwd(const void* view, const MokGemmTask* task, "
-        "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc);");
+        "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc, const mok::GemmCarry* carry);");
+PL_CALL(gemm_store, "mok_gemm_store",
+        "extern \"C\" __device__ void pipelink_call_gemm_store(const void* view, const MokGemmTask* task, const mok::AccFrag* acc);");
 PL_CALL(act_fwd, "mok_act_fwd",
         "extern \"C\" __device__ void pipelink_call_act_fwd(const void* view, const MokActTask* task, "
         "const MokCounters* counters, uint32_t* phase, const mok::AccFrag* acc);");

@@ -33,10 +33,12 @@
 #include <pipelink/stage.hpp>
 #ifndef PIPELINK_EMIT
 #include <type_traits>
+#include <utility>
 #include "../include/mok_device.hpp"
 
 extern "C" __device__ int pipelink_mok_gemm_depth();  // ring slots (2 or 4), bound at link time
-extern "C" __device__ int pipelink_mok_gemm_arena();  // byte offset of the ring in dynamic LDS
+extern "C" __device__ int pipelink_mok_gemm_head();   // byte offset of the rings' first two buffers + scale buffers in dynamic LDS
+extern "C" __device__ int pipelink_mok_gemm_arena();  // byte offset of the rings' other buffers
 
 extern __shared__ __attribute__((aligned(1024))) unsigned char pipelink_smem[];
 
@@ -81,12 +83,27 @@ struct Loader {
   int dst;                        // buffer-relative LDS byte offset of the wave's first group (both rings)
 };
 
-// LDS areas of one workgroup
+// LDS areas of one workgroup.  The first two buffers of each ring and the scale buffers (the
+// "head", claimed for the whole kernel) take the next tile's first loads while the current
+// tile's epilogue runs; the other buffers (the "arena", claimed for the GEMM phase only) share
+// their LDS with the epilogue's staging tile.
+//   head : X0 X1 W0 W1 | 4 x 1 KB weight scales | 2 x 4 KB routed-row scales
+//   arena: X2 .. X[DEPTH] | W2 .. W[DEPTH-1]
+constexpr int HEAD_BYTES = 4 * BUF_BYTES + WSCALE_BYTES + XSCALE_BYTES;
+template <int DEPTH>
 struct Rings {
-  unsigned char* x;       // DEPTH + 1 buffers
-  unsigned char* w;       // DEPTH buffers
-  unsigned char* wscale;  // 4 x 1 KB
-  unsigned char* xscale;  // 2 x 4 KB
+  unsigned char* head;
+  unsigned char* arena;
+  __device__ __forceinline__ Rings()
+      : head(pipelink_smem + pipelink_mok_gemm_head()), arena(pipelink_smem + pipelink_mok_gemm_arena()) {}
+  __device__ __forceinline__ unsigned char* x(int b) const {  // routed-row buffer b of DEPTH + 1
+    return b < 2 ? head + b * BUF_BYTES : arena + (b - 2) * BUF_BYTES;
+  }
+  __device__ __forceinline__ unsigned char* w(int b) const {  // weight buffer b of DEPTH
+    return b < 2 ? head + (2 + b) * BUF_BYTES : arena + (DEPTH - 1 + b - 2) * BUF_BYTES;
+  }
+  __device__ __forceinline__ unsigned char* wscale() const { return head + 4 * BUF_BYTES; }
+  __device__ __forceinline__ unsigned char* xscale() const { return head + 4 * BUF_BYTES + WSCALE_BYTES; }
 };
 
 __device__ __forceinline__ int swizzle(int row) { return (row >> 2) & 3; }
@@ -95,17 +112,17 @@ __device__ __forceinline__ int swizzle(int row) { return (row >> 2) & 3; }
 // go with slot j.  Scale loads go first so that they are older than tile loads of the same
 // step: the outstanding-load counts the waits use only count tile loads, which errs on the
 // side of waiting for more.  J8 is j % 8 where the caller knows it at compile time, else -1.
-template <int J8 = -1>
-__device__ __forceinline__ void issue_w(const Loader& ld, const Rings& r, int j, int buf) {
+template <int J8 = -1, int DEPTH>
+__device__ __forceinline__ void issue_w(const Loader& ld, const Rings<DEPTH>& r, int j, int buf) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t kbyte = (uint32_t)j * K_SLOT;
   const int j8 = J8 >= 0 ? J8 : (j & 7);
   // every eighth slot: 16 scale bytes of each routed row (this slot and the next seven)
-  if (j8 == 0) buf16_to_lds(ld.xsc, ld.xscsrc, kbyte >> 5, r.xscale + ((j >> 3) & 1) * (TILE_X * 16) + wave * 1024);
+  if (j8 == 0) buf16_to_lds(ld.xsc, ld.xscsrc, kbyte >> 5, r.xscale() + ((j >> 3) & 1) * (TILE_X * 16) + wave * 1024);
   // every second slot: the tile's weight scales of this pair, one row per thread
   if ((j8 & 1) == 0)
-    buf4_to_lds(ld.wsc, ld.wscsrc, (uint32_t)(j >> 1) * ld.wsc_pair_pitch, r.wscale + (j8 >> 1) * (TILE_W * 4) + wave * 256);
-  unsigned char* dst = r.w + buf * BUF_BYTES + ld.dst;
+    buf4_to_lds(ld.wsc, ld.wscsrc, (uint32_t)(j >> 1) * ld.wsc_pair_pitch, r.wscale() + (j8 >> 1) * (TILE_W * 4) + wave * 256);
+  unsigned char* dst = r.w(buf) + ld.dst;
   const uint32_t wslot = (uint32_t)j * ld.w_slot_pitch;
 #pragma unroll
   for (int i = 0; i < W_GROUPS; ++i) buf16_to_lds(ld.w, ld.wsrc[i], wslot, dst + i * 1024);
@@ -113,14 +130,38 @@ __device__ __forceinline__ void issue_w(const Loader& ld, const Rings& r, int j,
 
 // Issue the routed rows of slots j and j+1 (j even: the two halves of a 128-byte line) into
 // routed-row buffers buf0 and buf1, the two loads of a row group back to back.
-__device__ __forceinline__ void issue_x_pair(const Loader& ld, const Rings& r, int j, int buf0, int buf1) {
+template <int DEPTH>
+__device__ __forceinline__ void issue_x_pair(const Loader& ld, const Rings<DEPTH>& r, int j, int buf0, int buf1) {
   const uint32_t kbyte = (uint32_t)j * K_SLOT;
-  unsigned char* dst0 = r.x + buf0 * BUF_BYTES + ld.dst;
-  unsigned char* dst1 = r.x + buf1 * BUF_BYTES + ld.dst;
+  unsigned char* dst0 = r.x(buf0) + ld.dst;
+  unsigned char* dst1 = r.x(buf1) + ld.dst;
 #pragma unroll
   for (int i = 0; i < X_GROUPS; ++i) {
     buf16_to_lds(ld.x, ld.xsrc[i], kbyte, dst0 + i * 1024);
     buf16_to_lds(ld.x, ld.xsrc[i], kbyte + K_SLOT, dst1 + i * 1024);
+  }
+}
+
+// The same loads one at a time, for the steady-state steps that place every load between two
+// particular MFMAs.  Load L of the step that issues slot j (J8 = j % 8):
+//   even step: 0 routed-row scales (if J8 == 0), 1 weight scales, 2..9 routed rows (group (L-2)/2,
+//              half (L-2)%2, into routed-row buffers xb0 / xb1), 10..13 weight rows
+//   odd step:  0..3 weight rows
+template <bool ODD, int J8, int L, int DEPTH>
+__device__ __forceinline__ void issue_one(const Loader& ld, const Rings<DEPTH>& r, int j, int wbuf, int xb0, int xb1) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t kbyte = (uint32_t)j * K_SLOT;
+  constexpr int WL = ODD ? L : L - 10;  // weight group
+  if constexpr (!ODD && L == 0) {
+    if constexpr (J8 == 0) buf16_to_lds(ld.xsc, ld.xscsrc, kbyte >> 5, r.xscale() + ((j >> 3) & 1) * (TILE_X * 16) + wave * 1024);
+  } else if constexpr (!ODD && L == 1) {
+    static_assert(ODD || (J8 & 1) == 0, "even steps issue even slots");
+    buf4_to_lds(ld.wsc, ld.wscsrc, (uint32_t)(j >> 1) * ld.wsc_pair_pitch, r.wscale() + (J8 >> 1) * (TILE_W * 4) + wave * 256);
+  } else if constexpr (!ODD && L >= 2 && L < 10) {
+    constexpr int G = (L - 2) / 2, H = (L - 2) % 2;
+    buf16_to_lds(ld.x, ld.xsrc[G], kbyte + H * K_SLOT, r.x(H ? xb1 : xb0) + ld.dst + G * 1024);
+  } else if constexpr (WL >= 0 && WL < W_GROUPS) {
+    buf16_to_lds(ld.w, ld.wsrc[WL], (uint32_t)j * ld.w_slot_pitch, r.w(wbuf) + ld.dst + WL * 1024);
   }
 }
 
@@ -183,18 +224,30 @@ __device__ __forceinline__ void wait_loads_and_reads_dyn(int n) {
 // of the upper half use blocks 1 and 3, shifted down into bytes 0 and 2 where the MFMA's
 // op_sel picks them (0 in the pair's first slot, 2 in its second).  The routed rows' dwords
 // sit 16 bytes apart (a 4-way bank conflict on four small reads per pair).
-template <int J8 = -1>
+template <int J8 = -1, bool SHIFT = true>
 __device__ __forceinline__ void read_scales(int (&sx)[XFRAGS], int (&sw)[WFRAGS], const unsigned char* wscale,
                                             const unsigned char* xscale, int j, const int (&xscoff)[XFRAGS],
                                             const int (&wscoff)[WFRAGS], int half) {
   const int c = (J8 >= 0 ? J8 : (j & 7)) >> 1;
   const unsigned char* xbuf = xscale + ((j >> 3) & 1) * (TILE_X * 16);
 #pragma unroll
-  for (int b = 0; b < XFRAGS; ++b)
-    sx[b] = (int)(*reinterpret_cast<const uint32_t*>(xbuf + 4 * c + xscoff[b]) >> (8 * half));
+  for (int b = 0; b < XFRAGS; ++b) {
+    const uint32_t v = *reinterpret_cast<const uint32_t*>(xbuf + 4 * c + xscoff[b]);
+    sx[b] = (int)(SHIFT ? v >> (8 * half) : v);
+  }
   const unsigned char* wbuf = wscale + c * (TILE_W * 4);
 #pragma unroll
-  for (int a = 0; a < WFRAGS; ++a) sw[a] = (int)(*reinterpret_cast<const uint32_t*>(wbuf + wscoff[a]) >> (8 * half));
+  for (int a = 0; a < WFRAGS; ++a) {
+    const uint32_t v = *reinterpret_cast<const uint32_t*>(wbuf + wscoff[a]);
+    sw[a] = (int)(SHIFT ? v >> (8 * half) : v);
+  }
+}
+// second half of read_scales<.., false>
+__device__ __forceinline__ void shift_scales(int (&sx)[XFRAGS], int (&sw)[WFRAGS], int half) {
+#pragma unroll
+  for (int b = 0; b < XFRAGS; ++b) sx[b] = (int)((uint32_t)sx[b] >> (8 * half));
+#pragma unroll
+  for (int a = 0; a < WFRAGS; ++a) sw[a] = (int)((uint32_t)sw[a] >> (8 * half));
 }
 
 template <bool ODD>
@@ -208,73 +261,108 @@ __device__ __forceinline__ void mma_step(const Operands& o, const int (&sx)[XFRA
                                                                     sw[a], ODD ? 2 : 0, sx[b]);
 }
 
-template <int DEPTH>
-__device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmTask& t, AccFrag& acc) {
-  const int tid = threadIdx.x;
+// The gathered part of a tile's loader: routed row -> source row goes through row_token for
+// the gate/up op, a dependent global load.
+__device__ __forceinline__ void gather_rows(const MokGemmResidue& g, const MokGemmTask& t, GemmCarry& c) {
+  const int tid = fresh_tid();
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool gate_up = t.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
+  const MokMxView& act = gate_up ? g.x : g.hidden;
+  const int lrow = lane >> 2;
+  const int chunk = 16 * ((lane & 3) ^ swizzle(lrow));
+#pragma unroll
+  for (int i = 0; i < X_GROUPS; ++i) {
+    const int trow = (wave * X_GROUPS + i) * 16 + lrow;  // tile-local routed row
+    int row = t.row_begin + trow;
+    row = row < t.row_end ? row : t.row_end - 1;
+    const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
+    c.xsrc[i] = (uint32_t)src * (uint32_t)act.ld_q + chunk;
+  }
+  // routed-row scales: thread tid fetches row tid's 16-byte piece
+  int row = t.row_begin + tid;
+  row = row < t.row_end ? row : t.row_end - 1;
+  const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
+  c.xscsrc = (uint32_t)src * (uint32_t)act.ld_sc;
+}
+
+// Loader of a tile: lane -> (row lane/4 of a 16-row group, LDS position lane%4); it fetches the
+// chunk that belongs at that position.  Groups start at multiples of 16 rows, so the swizzle
+// of a row only depends on its place in the group.
+__device__ __forceinline__ Loader make_loader(const MokGemmResidue& g, const MokGemmTask& t, const GemmCarry& c) {
+  const int tid = fresh_tid();
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: resources chosen by it stay scalar
-  const int r32 = lane & 31;
-  const int half = lane >> 5;
   const bool gate_up = t.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
   const int expert = __builtin_amdgcn_readfirstlane(t.expert);
   const MokMxView& act = gate_up ? g.x : g.hidden;
+  Loader ld;
+  const int lrow = lane >> 2;
+  const int chunk = 16 * ((lane & 3) ^ swizzle(lrow));
+#pragma unroll
+  for (int i = 0; i < X_GROUPS; ++i) ld.xsrc[i] = c.xsrc[i];
+  ld.xscsrc = c.xscsrc;
+  ld.x = make_rsrc(act.q, (uint32_t)act.rows * (uint32_t)act.ld_q);
+  ld.xsc = make_rsrc(act.sc, (uint32_t)act.rows * (uint32_t)act.ld_sc);
+  ld.dst = wave * X_GROUPS * 1024;
+  static_assert(X_GROUPS == W_GROUPS, "one wave offset serves both rings");
+  const MokMxView& wv = gate_up ? (wave < WAVES / 2 ? g.w_gate : g.w_up) : g.w_down;
+#pragma unroll
+  for (int i = 0; i < W_GROUPS; ++i) {
+    const int wl = (wave * W_GROUPS + i) * 16 + lrow;  // tile-local weight row
+    int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
+    col = col < wv.rows ? col : wv.rows - 1;
+    ld.wsrc[i] = (uint32_t)col * (uint32_t)K_SLOT + chunk;  // weights are K-tiled: [K/64][rows][64]
+  }
+  ld.w = make_rsrc(wv.q + (int64_t)expert * wv.expert_pitch_q, (uint32_t)wv.rows * (uint32_t)wv.k);
+  ld.w_slot_pitch = (uint32_t)wv.rows * (uint32_t)K_SLOT;
+  // weight scales, slot-major [pair][row][4]: thread tid fetches tile row tid's dword
+  static_assert(THREADS == TILE_W, "one thread per weight row");
+  int col = t.col_begin + (gate_up ? (tid & (TILE_W / 2 - 1)) : tid);
+  col = col < wv.rows ? col : wv.rows - 1;
+  ld.wsc = make_rsrc(wv.sc + (int64_t)expert * wv.expert_pitch_sc,
+                     (uint32_t)((wv.k + K_PAIR - 1) / K_PAIR) * (uint32_t)wv.rows * 4u);
+  ld.wscsrc = (uint32_t)col * 4u;
+  ld.wsc_pair_pitch = (uint32_t)wv.rows * 4u;
+  return ld;
+}
+
+// The schedule plays steps -DEPTH .. -1 before a tile's first MFMA: step u issues the weight
+// rows of slot u + DEPTH and, on even u, the routed rows of slots u + DEPTH and u + DEPTH + 1.
+// The first two of those steps only touch head buffers: `prefetch` issues them, and may run
+// while the previous tile's epilogue still uses the arena.
+template <int DEPTH>
+__device__ __forceinline__ void issue_prologue_step(const Loader& ld, const Rings<DEPTH>& r, int s, int n) {
+  if (s < n) {
+    if ((s & 1) == 0) issue_x_pair(ld, r, s, s, s + 1);
+    issue_w(ld, r, s, s);
+  }
+}
+
+template <int DEPTH>
+__device__ __forceinline__ void prefetch(const MokGemmResidue& g, const MokGemmTask& t, GemmCarry& c) {
+  gather_rows(g, t, c);
+  const Loader ld = make_loader(g, t, c);
+  const Rings<DEPTH> r;
+  const int n = (t.op == MOK_GEMM_FWD_ROUTED_GATE_UP ? g.x.k : g.hidden.k) / K_SLOT;
+  issue_prologue_step(ld, r, 0, n);
+  issue_prologue_step(ld, r, 1, n);
+}
+
+template <int DEPTH>
+__device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmTask& t, AccFrag& acc,
+                                         const GemmCarry& carry) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r32 = lane & 31;
+  const int half = lane >> 5;
+  const bool gate_up = t.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
+  const MokMxView& act = gate_up ? g.x : g.hidden;
   const int n = act.k / K_SLOT;  // the host rejects a contraction length that is not a multiple of 64
   constexpr int XDEPTH = DEPTH + 1;
-  Rings r;
-  r.x = pipelink_smem + pipelink_mok_gemm_arena();
-  r.w = r.x + XDEPTH * BUF_BYTES;
-  r.wscale = r.w + DEPTH * BUF_BYTES;
-  r.xscale = r.wscale + WSCALE_BYTES;
-
-  // ---- loader addresses (fixed for the tile) ---------------------------------------
-  // lane -> (row lane/4 of a 16-row group, LDS position lane%4); it fetches the chunk that
-  // belongs at that position.  Groups start at multiples of 16 rows, so the swizzle of a row
-  // only depends on its place in the group.
-  Loader ld;
-  {
-    const int lrow = lane >> 2;
-    const int chunk = 16 * ((lane & 3) ^ swizzle(lrow));
-#pragma unroll
-    for (int i = 0; i < X_GROUPS; ++i) {
-      const int trow = (wave * X_GROUPS + i) * 16 + lrow;  // tile-local routed row
-      int row = t.row_begin + trow;
-      row = row < t.row_end ? row : t.row_end - 1;
-      const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
-      ld.xsrc[i] = (uint32_t)src * (uint32_t)act.ld_q + chunk;
-    }
-    ld.x = make_rsrc(act.q, (uint32_t)act.rows * (uint32_t)act.ld_q);
-    ld.dst = wave * X_GROUPS * 1024;
-    static_assert(X_GROUPS == W_GROUPS, "one wave offset serves both rings");
-    const MokMxView& wv = gate_up ? (wave < WAVES / 2 ? g.w_gate : g.w_up) : g.w_down;
-#pragma unroll
-    for (int i = 0; i < W_GROUPS; ++i) {
-      const int wl = (wave * W_GROUPS + i) * 16 + lrow;  // tile-local weight row
-      int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
-      col = col < wv.rows ? col : wv.rows - 1;
-      ld.wsrc[i] = (uint32_t)col * (uint32_t)K_SLOT + chunk;  // weights are K-tiled: [K/64][rows][64]
-    }
-    ld.w = make_rsrc(wv.q + (int64_t)expert * wv.expert_pitch_q, (uint32_t)wv.rows * (uint32_t)wv.k);
-    ld.w_slot_pitch = (uint32_t)wv.rows * (uint32_t)K_SLOT;
-    // routed-row scales: thread tid fetches row tid's 16-byte piece
-    {
-      int row = t.row_begin + tid;
-      row = row < t.row_end ? row : t.row_end - 1;
-      const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
-      ld.xsc = make_rsrc(act.sc, (uint32_t)act.rows * (uint32_t)act.ld_sc);
-      ld.xscsrc = (uint32_t)src * (uint32_t)act.ld_sc;
-    }
-    // weight scales, slot-major [pair][row][4]: thread tid fetches tile row tid's dword
-    {
-      static_assert(THREADS == TILE_W, "one thread per weight row");
-      const MokMxView& sv = gate_up ? (wave < WAVES / 2 ? g.w_gate : g.w_up) : g.w_down;
-      int col = t.col_begin + (gate_up ? (tid & (TILE_W / 2 - 1)) : tid);
-      col = col < sv.rows ? col : sv.rows - 1;
-      ld.wsc = make_rsrc(sv.sc + (int64_t)expert * sv.expert_pitch_sc,
-                         (uint32_t)((sv.k + K_PAIR - 1) / K_PAIR) * (uint32_t)sv.rows * 4u);
-      ld.wscsrc = (uint32_t)col * 4u;
-      ld.wsc_pair_pitch = (uint32_t)sv.rows * 4u;
-    }
-  }
+  const Rings<DEPTH> r;
+  const Loader ld = make_loader(g, t, carry);
 
   // ---- per-fragment LDS read offsets (first block) ------------------------------------
   int xoff[XFRAGS], woff[WFRAGS], xscoff[XFRAGS], wscoff[WFRAGS];
@@ -309,15 +397,9 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   constexpr int STEADY = (DEPTH - 2) * W_LOADS + (DEPTH - 2) / 2 * X_LOADS;  // DEPTH is even
   static_assert(DEPTH % 2 == 0, "routed-row pairs are issued on even steps");
 
-  // ---- prologue: steps -DEPTH .. -1 of the schedule, then slot 0's operands --------------
+  // ---- rest of the prologue (slots 0 and 1 were issued by `prefetch`), then slot 0's operands
 #pragma unroll
-  for (int u = -DEPTH; u < 0; ++u) {
-    const int s = u + DEPTH;
-    if (s < n) {
-      if ((s & 1) == 0) issue_x_pair(ld, r, s, s, s + 1);
-      issue_w(ld, r, s, s);
-    }
-  }
+  for (int s2 = 2; s2 < DEPTH; ++s2) issue_prologue_step(ld, r, s2, n);
   {  // slot 0: younger loads are those of prologue steps 1-DEPTH .. -1
     int younger = 0;
 #pragma unroll
@@ -327,8 +409,8 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   wg_barrier();
   Operands even, odd;
   int sx[XFRAGS], sw[WFRAGS], sxn[XFRAGS], swn[WFRAGS];
-  read_operands(even, r.x, r.w, xoff, woff);
-  read_scales(sx, sw, r.wscale, r.xscale, 0, xscoff, wscoff, half);
+  read_operands(even, r.x(0), r.w(0), xoff, woff);
+  read_scales(sx, sw, r.wscale(), r.xscale(), 0, xscoff, wscoff, half);
 
   // Step j multiplies slot j (already in registers) while it fetches slot j+1's operands from
   // LDS; the barrier in front says slot j+1 has landed for every wave and every wave holds
@@ -356,27 +438,49 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       wait_loads_and_reads<STEADY>();
       wg_barrier();
       // slot j+S's buffers are free; so is the routed-row buffer before it (freed a step ago)
-      const int xprev = xnext(xb, XDEPTH - 1);
-      if (!ODD) issue_x_pair(ld, r, j + S + DEPTH, xprev, xb);
-      issue_w<(S + DEPTH) & 7>(ld, r, j + S + DEPTH, S % DEPTH);
+      const int xprev = xnext(xb, XDEPTH - 1), xcur = xb;
       xb = xnext(xb, 1);
-      read_operands(next, r.x + xb * BUF_BYTES, r.w + ((S + 1) % DEPTH) * BUF_BYTES, xoff, woff);
-      if (ODD) read_scales<(S + 1) & 7>(sxn, swn, r.wscale, r.xscale, j + S + 1, xscoff, wscoff, half);
-      mma_step<ODD>(cur, sx, sw, acc);
-      // issue order inside the step: an MFMA first (the pipe must not drain behind the
-      // barrier), the global loads spread over the first MFMAs, the LDS reads over the rest
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-      __builtin_amdgcn_sched_group_barrier(0x010, 3, 0);  // VMEM: the scale loads and the first tile load
-#pragma unroll
-      for (int i = 1; i < 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x010, ODD ? 1 : 2, 0);  // VMEM
-      }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);  // LDS reads
-      }
+      const unsigned char* xnew = r.x(xb);
+      const unsigned char* wnew = r.w((S + 1) % DEPTH);
+      // The step, MFMA by MFMA.  One LDS unit and one texture-address unit serve the four
+      // waves: an LDS read costs the unit about 8 cycles and a 1 KB load about 16, so a wave
+      // puts at most two reads and one load between two 64-cycle MFMAs, or the MFMA behind
+      // them issues late.  The reads sit in the first 12 of the 16 places (the barrier of the
+      // next step wants them back), the loads are spread over all of them.  The scheduler may
+      // not move anything from one place to another.
+      auto place = [&](auto I_) {
+        constexpr int I = decltype(I_)::value;
+        constexpr int A = I / XFRAGS, B = I % XFRAGS;
+        acc.v[A][B] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cur.w[A], cur.x[B], acc.v[A][B], 0, 0, ODD ? 2 : 0,
+                                                                      sw[A], ODD ? 2 : 0, sx[B]);
+        __builtin_amdgcn_sched_barrier(0);  // the MFMA goes first: the pipe is what must not wait
+        // operand fragment K of the next slot: routed rows first, they are needed by the first MFMAs
+        constexpr int K = I == 0 ? 0 : I == 1 ? 1 : I == 3 ? 2 : I == 4 ? 3 : I == 6 ? 4 : I == 7 ? 5 : I == 9 ? 6 : I == 10 ? 7 : -1;
+        if constexpr (K >= 0 && K < XFRAGS) next.x[K] = read_frag(xnew, xoff[K]);
+        if constexpr (K >= XFRAGS) next.w[K - XFRAGS] = read_frag(wnew, woff[K - XFRAGS]);
+        // next pair's scale dwords: read here, shifted into place three MFMAs later, when they have arrived
+        if constexpr (ODD && I == 11) read_scales<(S + 1) & 7, false>(sxn, swn, r.wscale(), r.xscale(), j + S + 1, xscoff, wscoff, half);
+        if constexpr (ODD && I == 14) shift_scales(sxn, swn, half);
+        if constexpr (!ODD) issue_one<false, (S + DEPTH) & 7, I>(ld, r, j + S + DEPTH, S % DEPTH, xprev, xcur);
+        if constexpr (ODD && I % 4 == 1) issue_one<true, (S + DEPTH) & 7, I / 4>(ld, r, j + S + DEPTH, S % DEPTH, xprev, xcur);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      place(std::integral_constant<int, 0>{});
+      place(std::integral_constant<int, 1>{});
+      place(std::integral_constant<int, 2>{});
+      place(std::integral_constant<int, 3>{});
+      place(std::integral_constant<int, 4>{});
+      place(std::integral_constant<int, 5>{});
+      place(std::integral_constant<int, 6>{});
+      place(std::integral_constant<int, 7>{});
+      place(std::integral_constant<int, 8>{});
+      place(std::integral_constant<int, 9>{});
+      place(std::integral_constant<int, 10>{});
+      place(std::integral_constant<int, 11>{});
+      place(std::integral_constant<int, 12>{});
+      place(std::integral_constant<int, 13>{});
+      place(std::integral_constant<int, 14>{});
+      place(std::integral_constant<int, 15>{});
       __builtin_amdgcn_sched_barrier(0);
       if (ODD) {
 #pragma unroll
@@ -411,13 +515,13 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
     }
     xb = xnext(xb, 1);
     wb = wb + 1 == DEPTH ? 0 : wb + 1;
-    read_operands(next, r.x + xb * BUF_BYTES, r.w + wb * BUF_BYTES, xoff, woff);
+    read_operands(next, r.x(xb), r.w(wb), xoff, woff);
   };
   for (; j + 1 < n; j += 2) {
     advance(j, odd);
     mma_step<false>(even, sx, sw, acc);
     advance(j + 1, even);
-    read_scales(sxn, swn, r.wscale, r.xscale, j + 2, xscoff, wscoff, half);
+    read_scales(sxn, swn, r.wscale(), r.xscale(), j + 2, xscoff, wscoff, half);
     mma_step<true>(odd, sx, sw, acc);
 #pragma unroll
     for (int b = 0; b < XFRAGS; ++b) sx[b] = sxn[b];
@@ -428,9 +532,11 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   wg_barrier();  // every wave holds its last operands in registers: the ring is free
 }
 
-// bf16 epilogue of the down op.  The accumulator is transposed through the (now idle) ring so
-// that the global stores are 16 bytes per lane and 512 contiguous bytes per routed row.  A
-// ring too small for the whole tile stages the two 128-row halves one after the other.
+// bf16 epilogue of the down op.  The accumulator is transposed through the arena buffers (idle
+// by now; the head may already hold the next tile's first slots) so that the global stores
+// are 16 bytes per lane and 512 contiguous bytes per routed row; an arena too small for the
+// whole tile stages the two 128-row halves one after the other.  An arena that cannot hold
+// half a tile (depth 2) falls back to 8-byte stores straight from the registers.
 constexpr int Y_PITCH = TILE_W * 2 + 16;  // bytes per staged row: 256 bf16 + pad against bank conflicts
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -443,68 +549,107 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 
 template <int DEPTH>
 __device__ __forceinline__ void store_down(const MokGemmResidue& g, const MokGemmTask& t, const AccFrag& acc) {
-  constexpr int RING_BYTES = (2 * DEPTH + 1) * BUF_BYTES + WSCALE_BYTES + XSCALE_BYTES;
-  constexpr int PASSES = TILE_X * Y_PITCH <= RING_BYTES ? 1 : 2;
-  constexpr int ROWS = TILE_X / PASSES;  // rows staged per pass
-  static_assert(ROWS * Y_PITCH <= RING_BYTES, "half a tile must fit the ring");
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  unsigned char* stage = pipelink_smem + pipelink_mok_gemm_arena();
-  const int chunk = lane & 31;                                  // 8 columns = 16 bytes
-  const bool col_ok = t.col_begin + chunk * 8 < g.w_down.rows;  // column extents are multiples of 32
+  constexpr int ARENA_BYTES = (2 * DEPTH - 3) * BUF_BYTES;
+  const int tid = fresh_tid();
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  if constexpr (ARENA_BYTES < TILE_X / 2 * Y_PITCH) {
 #pragma unroll
-  for (int pass = 0; pass < PASSES; ++pass) {
-    if (PASSES == 1 || wave_x(wave) == pass) {
+    for (int b = 0; b < XFRAGS; ++b) {
+      const int row = t.row_begin + xrow0(wave, b) + (lane & 31);
 #pragma unroll
-      for (int b = 0; b < XFRAGS; ++b) {
-        unsigned char* rowp = stage + (xrow0(wave, b) - pass * ROWS + (lane & 31)) * Y_PITCH;
+      for (int a = 0; a < WFRAGS; ++a) {
 #pragma unroll
-        for (int a = 0; a < WFRAGS; ++a) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int col = wrow0(wave, a) + 8 * q + 4 * (lane >> 5);
+        for (int q = 0; q < 4; ++q) {
+          const int col = t.col_begin + wrow0(wave, a) + 8 * q + 4 * (lane >> 5);
+          if (row < t.row_end && col < g.w_down.rows) {
             uint2 pk;
             pk.x = pack_bf16x2(acc.v[a][b][4 * q + 0], acc.v[a][b][4 * q + 1]);
             pk.y = pack_bf16x2(acc.v[a][b][4 * q + 2], acc.v[a][b][4 * q + 3]);
-            *reinterpret_cast<uint2*>(rowp + col * 2) = pk;
+            *reinterpret_cast<uint2*>(g.y + (int64_t)row * g.ld_y + col) = pk;
           }
         }
       }
     }
-    __syncthreads();
-#pragma unroll 4
-    for (int it = 0; it < ROWS / WAVES / 2; ++it) {
-      const int srow = wave * (ROWS / WAVES) + it * 2 + (lane >> 5);
-      const int row = t.row_begin + pass * ROWS + srow;
-      if (row < t.row_end && col_ok) {
-        const uint4 v = *reinterpret_cast<const uint4*>(stage + srow * Y_PITCH + chunk * 16);
-        *reinterpret_cast<uint4*>(g.y + (int64_t)row * g.ld_y + t.col_begin + chunk * 8) = v;
+  } else {
+    constexpr int PASSES = TILE_X * Y_PITCH <= ARENA_BYTES ? 1 : 2;
+    constexpr int ROWS = TILE_X / PASSES;  // rows staged per pass
+    unsigned char* stage = pipelink_smem + pipelink_mok_gemm_arena();
+    const int chunk = lane & 31;                                  // 8 columns = 16 bytes
+    const bool col_ok = t.col_begin + chunk * 8 < g.w_down.rows;  // column extents are multiples of 32
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass) {
+      if (PASSES == 1 || wave_x(wave) == pass) {
+#pragma unroll
+        for (int b = 0; b < XFRAGS; ++b) {
+          unsigned char* rowp = stage + (xrow0(wave, b) - pass * ROWS + (lane & 31)) * Y_PITCH;
+#pragma unroll
+          for (int a = 0; a < WFRAGS; ++a) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int col = wrow0(wave, a) + 8 * q + 4 * (lane >> 5);
+              uint2 pk;
+              pk.x = pack_bf16x2(acc.v[a][b][4 * q + 0], acc.v[a][b][4 * q + 1]);
+              pk.y = pack_bf16x2(acc.v[a][b][4 * q + 2], acc.v[a][b][4 * q + 3]);
+              *reinterpret_cast<uint2*>(rowp + col * 2) = pk;
+            }
+          }
+        }
       }
+      __syncthreads();
+#pragma unroll 4
+      for (int it = 0; it < ROWS / WAVES / 2; ++it) {
+        const int srow = wave * (ROWS / WAVES) + it * 2 + (lane >> 5);
+        const int row = t.row_begin + pass * ROWS + srow;
+        if (row < t.row_end && col_ok) {
+          const uint4 v = *reinterpret_cast<const uint4*>(stage + srow * Y_PITCH + chunk * 16);
+          *reinterpret_cast<uint4*>(g.y + (int64_t)row * g.ld_y + t.col_begin + chunk * 8) = v;
+        }
+      }
+      __syncthreads();  // the arena is reused by the next pass or the next tile's loads
     }
-    __syncthreads();  // the ring is reused by the next pass or the next tile's loads
   }
-}
-
-template <int DEPTH>
-__device__ __forceinline__ void run(const MokGemmResidue& g, const MokGemmTask& t, AccFrag& acc) {
-  mainloop<DEPTH>(g, t, acc);
-  if (t.op == MOK_GEMM_FWD_ROUTED_DOWN) store_down<DEPTH>(g, t, acc);
 }
 
 }  // namespace mok_gemm_owner
 
 extern "C" __device__ void mok_gemm_init(const void* view) { (void)view; }
 
-// Runs the mainloop of one tile.  For the gate/up op the fp32 accumulator is left in *acc
-// for the activation owner; for the down op it is rounded to bf16 and stored here.
+static __device__ __forceinline__ const MokGemmResidue& mok_gemm_residue(const void* view) {
+  return *static_cast<const MokGemmResidue*>(static_cast<const pipelink_host_view*>(view)->residue);
+}
+
+// Starts the loads of a tile's first two slots and leaves the gathered row offsets in *carry.
+// Only touches the head buffers: the caller may run it between the previous tile's mainloop
+// and that tile's epilogue.
+extern "C" __device__ void mok_gemm_prefetch(const void* view, const MokGemmTask* task, mok::GemmCarry* carry) {
+  const auto& g = mok_gemm_residue(view);
+  switch (pipelink_mok_gemm_depth()) {  // a link-time constant: one case survives
+    case 2: mok_gemm_owner::prefetch<2>(g, *task, *carry); break;
+    default: mok_gemm_owner::prefetch<4>(g, *task, *carry); break;
+  }
+}
+
+// Runs the mainloop of one tile whose prefetch has been issued (same task, same carry) and
+// leaves the fp32 accumulator in *acc: for the activation owner (gate/up op) or for
+// mok_gemm_store (down op).
 extern "C" __device__ void mok_gemm_fwd(const void* view, const MokGemmTask* task, const MokCounters* counters,
-                                        uint32_t* phase, mok::AccFrag* acc) {
+                                        uint32_t* phase, mok::AccFrag* acc, const mok::GemmCarry* carry) {
   (void)counters;
   (void)phase;
-  const auto& g = *static_cast<const MokGemmResidue*>(static_cast<const pipelink_host_view*>(view)->residue);
-  switch (pipelink_mok_gemm_depth()) {  // a link-time constant: one case survives
-    case 2: mok_gemm_owner::run<2>(g, *task, *acc); break;
-    default: mok_gemm_owner::run<4>(g, *task, *acc); break;
+  const auto& g = mok_gemm_residue(view);
+  switch (pipelink_mok_gemm_depth()) {
+    case 2: mok_gemm_owner::mainloop<2>(g, *task, *acc, *carry); break;
+    default: mok_gemm_owner::mainloop<4>(g, *task, *acc, *carry); break;
+  }
+}
+
+// Down op only: rounds the accumulator to bf16 and stores the tile of y.
+extern "C" __device__ void mok_gemm_store(const void* view, const MokGemmTask* task, const mok::AccFrag* acc) {
+  const auto& g = mok_gemm_residue(view);
+  switch (pipelink_mok_gemm_depth()) {
+    case 2: mok_gemm_owner::store_down<2>(g, *task, *acc); break;
+    default: mok_gemm_owner::store_down<4>(g, *task, *acc); break;
   }
 }
 #else  // PIPELINK_EMIT: host-evaluated annotations only
@@ -516,14 +661,24 @@ PL_PARAMS(MokGemmResidue);
 PL_TOPOLOGY(true, "static");
 PL_VARIANT(0, {{"pipelink_mok_precision", 1}});  // MXFP8 (campaigns/mok/port/include/mok_abi.h: MOK_PRECISION_MXFP8)
 PL_EXPORT(mok_gemm_init, mok_gemm_init, "extern \"C\" __device__ void mok_gemm_init(const void* view);");
+PL_EXPORT(mok_gemm_prefetch, mok_gemm_prefetch,
+          "extern \"C\" __device__ void mok_gemm_prefetch(const void* view, const MokGemmTask* task, mok::GemmCarry* carry);");
 PL_EXPORT(mok_gemm_fwd, mok_gemm_fwd,
           "extern \"C\" __device__ void mok_gemm_fwd(const void* view, const MokGemmTask* task, "
-          "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc);");
+          "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc, const mok::GemmCarry* carry);");
+PL_EXPORT(mok_gemm_store, mok_gemm_store,
+          "extern \"C\" __device__ void mok_gemm_store(const void* view, const MokGemmTask* task, const mok::AccFrag* acc);");
 PL_SERVE(gemm_init, "mok_gemm_init");
+PL_SERVE(gemm_prefetch, "mok_gemm_prefetch");
 PL_SERVE(gemm_fwd, "mok_gemm_fwd");
-// per unit of depth one 16 KB weight buffer and one 16 KB routed-row buffer; fixed: the extra routed-row
-// buffer, four 1 KB buffers of weight scales, two 4 KB buffers of routed-row scales
-PL_CLAIM_RING("pipelink_mok_gemm_arena", "smem", 16384 + 12288, "pipelink_mok_gemm_depth", 32768, 1024, "phase:instr_gemm");
+PL_SERVE(gemm_store, "mok_gemm_store");
+// head, live for the whole kernel: the first two 16 KB buffers of the routed-row ring and of the weight
+// ring, four 1 KB buffers of weight scales, two 4 KB buffers of routed-row scales
+PL_CLAIM("pipelink_mok_gemm_head", "smem", 4 * 16384 + 4096 + 8192, 1024, "kernel");
+// arena, live during the GEMM phase: the other buffers of the two rings -- depth + 1 - 2 routed-row
+// buffers and depth - 2 weight buffers, (2 * depth - 3) x 16 KB
+PL_CLAIM_RING("pipelink_mok_gemm_arena", "smem", -3 * 16384, "pipelink_mok_gemm_depth", 32768, 1024, "phase:instr_gemm");
+PL_USES("pipelink_mok_gemm_head");
 PL_USES("pipelink_mok_gemm_depth");
 PL_USES("pipelink_mok_gemm_arena");
 PL_FACT("mok.gemm.TILE_X", 256);

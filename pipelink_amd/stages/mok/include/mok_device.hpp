@@ -39,6 +39,14 @@ struct AccFrag {
   v16f v[WFRAGS][XFRAGS];
 };
 
+// What the GEMM owner's prefetch export hands to its forward export for the same tile: the
+// lane's gathered routed-row offsets (they cost a dependent global load, which the prefetch
+// takes off the forward call's critical path).  Opaque to the other stages.
+struct GemmCarry {
+  uint32_t xsrc[TILE_X / 16 / (THREADS / 64)];
+  uint32_t xscsrc;
+};
+
 __device__ __forceinline__ int wave_w(int wave) { return wave & 1; }
 __device__ __forceinline__ int wave_x(int wave) { return wave >> 1; }
 // first tile-local weight row of fragment a for this wave (rows [0,128) | [128,256))
@@ -57,6 +65,15 @@ __device__ __forceinline__ void load16_to_lds(const uint8_t* g, unsigned char* l
 // 4 bytes per lane, lane i lands at lds + 4*i
 __device__ __forceinline__ void load4_to_lds(const uint8_t* g, unsigned char* lds) {
   __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)lds, 4, 0, 0);
+}
+
+// threadIdx.x as a value the compiler cannot merge with an earlier copy: code that runs after
+// a register-hungry loop derives its lane indices from this, so they are computed where they
+// are used instead of being kept (spilled) across the loop.
+__device__ __forceinline__ int fresh_tid() {
+  int t = threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
 }
 
 __device__ __forceinline__ float bf16_round(float x) {
