@@ -128,38 +128,42 @@ __device__ __forceinline__ void issue_w(const Loader& ld, const Rings<DEPTH>& r,
   for (int i = 0; i < W_GROUPS; ++i) buf16_to_lds(ld.w, ld.wsrc[i], wslot, dst + i * 1024);
 }
 
-// Issue the routed rows of slots j and j+1 (j even: the two halves of a 128-byte line) into
-// routed-row buffers buf0 and buf1, the two loads of a row group back to back.
-template <int DEPTH>
-__device__ __forceinline__ void issue_x_pair(const Loader& ld, const Rings<DEPTH>& r, int j, int buf0, int buf1) {
+// Issue row groups G0 .. G1-1 of the routed rows of slots j and j+1 (j even: the two halves of a
+// 128-byte line) into routed-row buffers buf0 and buf1, the two loads of a row group back to back.
+template <int G0, int G1, int DEPTH>
+__device__ __forceinline__ void issue_x_groups(const Loader& ld, const Rings<DEPTH>& r, int j, int buf0, int buf1) {
   const uint32_t kbyte = (uint32_t)j * K_SLOT;
   unsigned char* dst0 = r.x(buf0) + ld.dst;
   unsigned char* dst1 = r.x(buf1) + ld.dst;
 #pragma unroll
-  for (int i = 0; i < X_GROUPS; ++i) {
+  for (int i = G0; i < G1; ++i) {
     buf16_to_lds(ld.x, ld.xsrc[i], kbyte, dst0 + i * 1024);
     buf16_to_lds(ld.x, ld.xsrc[i], kbyte + K_SLOT, dst1 + i * 1024);
   }
 }
 
 // The same loads one at a time, for the steady-state steps that place every load between two
-// particular MFMAs.  Load L of the step that issues slot j (J8 = j % 8):
-//   even step: 0 routed-row scales (if J8 == 0), 1 weight scales, 2..9 routed rows (group (L-2)/2,
-//              half (L-2)%2, into routed-row buffers xb0 / xb1), 10..13 weight rows
-//   odd step:  0..3 weight rows
+// particular MFMAs.  Load L of the step that issues weight slot j (J8 = j % 8); the routed rows
+// belong to the pair of slots that starts at j (even step) or at j - 1 (odd step) and go into
+// routed-row buffers xb0 / xb1:
+//   even step: 0 routed-row scales (if J8 == 0), 1 weight scales, 2..5 routed rows (group (L-2)/2,
+//              half (L-2)%2), 6..9 weight rows
+//   odd step:  0..3 routed rows (group 2 + L/2, half L%2), 4..7 weight rows
 template <bool ODD, int J8, int L, int DEPTH>
 __device__ __forceinline__ void issue_one(const Loader& ld, const Rings<DEPTH>& r, int j, int wbuf, int xb0, int xb1) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t kbyte = (uint32_t)j * K_SLOT;
-  constexpr int WL = ODD ? L : L - 10;  // weight group
+  constexpr int XL = ODD ? L : L - 2;       // routed-row load 0..3 of this step
+  constexpr int WL = ODD ? L - 4 : L - 6;   // weight group
   if constexpr (!ODD && L == 0) {
     if constexpr (J8 == 0) buf16_to_lds(ld.xsc, ld.xscsrc, kbyte >> 5, r.xscale() + ((j >> 3) & 1) * (TILE_X * 16) + wave * 1024);
   } else if constexpr (!ODD && L == 1) {
     static_assert(ODD || (J8 & 1) == 0, "even steps issue even slots");
     buf4_to_lds(ld.wsc, ld.wscsrc, (uint32_t)(j >> 1) * ld.wsc_pair_pitch, r.wscale() + (J8 >> 1) * (TILE_W * 4) + wave * 256);
-  } else if constexpr (!ODD && L >= 2 && L < 10) {
-    constexpr int G = (L - 2) / 2, H = (L - 2) % 2;
-    buf16_to_lds(ld.x, ld.xsrc[G], kbyte + H * K_SLOT, r.x(H ? xb1 : xb0) + ld.dst + G * 1024);
+  } else if constexpr (XL >= 0 && XL < 4) {
+    constexpr int G = (ODD ? 2 : 0) + XL / 2, H = XL % 2;
+    const uint32_t kpair = ODD ? kbyte - K_SLOT : kbyte;  // the pair's first slot
+    buf16_to_lds(ld.x, ld.xsrc[G], kpair + H * K_SLOT, r.x(H ? xb1 : xb0) + ld.dst + G * 1024);
   } else if constexpr (WL >= 0 && WL < W_GROUPS) {
     buf16_to_lds(ld.w, ld.wsrc[WL], (uint32_t)j * ld.w_slot_pitch, r.w(wbuf) + ld.dst + WL * 1024);
   }
@@ -216,6 +220,7 @@ __device__ __forceinline__ void wait_loads_and_reads_dyn(int n) {
     case 12: wait_loads_and_reads<12>(); break;
     case 16: wait_loads_and_reads<16>(); break;
     case 20: wait_loads_and_reads<20>(); break;
+    case 24: wait_loads_and_reads<24>(); break;
     default: wait_loads_and_reads<0>(); break;  // waiting for everything is always right
   }
 }
@@ -327,16 +332,54 @@ __device__ __forceinline__ Loader make_loader(const MokGemmResidue& g, const Mok
   return ld;
 }
 
-// The schedule plays steps -DEPTH .. -1 before a tile's first MFMA: step u issues the weight
-// rows of slot u + DEPTH and, on even u, the routed rows of slots u + DEPTH and u + DEPTH + 1.
-// The first two of those steps only touch head buffers: `prefetch` issues them, and may run
-// while the previous tile's epilogue still uses the arena.
+// Loads of schedule step u (u < 0: before a tile's first MFMA), in this order: [scale loads]
+// [routed rows] [weight rows of slot u + DEPTH].  With DEPTH >= 4 the routed rows of a pair of
+// slots are split over two steps, so that every step issues the same 8 tile loads: groups 0-1
+// of the pair that starts at slot u + DEPTH on even u, groups 2-3 of the same pair on the odd
+// step after it.  With DEPTH == 2 the whole pair is issued on the even step.  Steps -DEPTH and
+// 1 - DEPTH only touch head buffers: `prefetch` issues them, and may run while the previous
+// tile's epilogue still uses the arena.
 template <int DEPTH>
-__device__ __forceinline__ void issue_prologue_step(const Loader& ld, const Rings<DEPTH>& r, int s, int n) {
-  if (s < n) {
-    if ((s & 1) == 0) issue_x_pair(ld, r, s, s, s + 1);
-    issue_w(ld, r, s, s);
+__device__ __forceinline__ void issue_step(const Loader& ld, const Rings<DEPTH>& r, int u, int n, int xb0, int xb1, int wb) {
+  constexpr bool SPLIT = DEPTH >= 4;
+  const int s = u + DEPTH;
+  const int pair = (u & 1) ? s - 1 : s;
+  if (pair < n) {
+    if (!SPLIT) {
+      if ((u & 1) == 0) issue_x_groups<0, X_GROUPS>(ld, r, pair, xb0, xb1);
+    } else if ((u & 1) == 0) {
+      issue_x_groups<0, X_GROUPS / 2>(ld, r, pair, xb0, xb1);
+    } else {
+      issue_x_groups<X_GROUPS / 2, X_GROUPS>(ld, r, pair, xb0, xb1);
+    }
   }
+  if (s < n) issue_w(ld, r, s, wb);
+}
+// tile loads issue_step(u) issues: routed rows, weight rows
+template <int DEPTH>
+__device__ __forceinline__ int x_loads_in(int u, int n) {
+  const int s = u + DEPTH;
+  const int pair = (u & 1) ? s - 1 : s;
+  if (pair >= n) return 0;
+  return DEPTH >= 4 ? X_LOADS / 2 : ((u & 1) == 0 ? X_LOADS : 0);
+}
+template <int DEPTH>
+__device__ __forceinline__ int w_loads_in(int u, int n) { return u + DEPTH < n ? W_LOADS : 0; }
+// Tile loads that may still be outstanding when slot `slot` is needed and steps up to `last`
+// have been issued (step t waits for slot t+1 with last = t-1; the prologue waits for slot 0
+// with last = -1).  The slot's weight rows are the last loads of step slot-DEPTH; its routed
+// rows come no later, except that with split pairs groups 2-3 of an even slot are issued at
+// the start of step slot+1-DEPTH.
+template <int DEPTH>
+__device__ __forceinline__ int loads_younger_than_slot(int slot, int last, int n) {
+  int younger = 0;
+  int first = slot + 1 - DEPTH;  // first step all of whose loads are younger
+  if (DEPTH >= 4 && (slot & 1) == 0) {
+    younger += w_loads_in<DEPTH>(first, n);
+    ++first;
+  }
+  for (int u = first; u <= last; ++u) younger += x_loads_in<DEPTH>(u, n) + w_loads_in<DEPTH>(u, n);
+  return younger;
 }
 
 template <int DEPTH>
@@ -345,8 +388,8 @@ __device__ __forceinline__ void prefetch(const MokGemmResidue& g, const MokGemmT
   const Loader ld = make_loader(g, t, c);
   const Rings<DEPTH> r;
   const int n = (t.op == MOK_GEMM_FWD_ROUTED_GATE_UP ? g.x.k : g.hidden.k) / K_SLOT;
-  issue_prologue_step(ld, r, 0, n);
-  issue_prologue_step(ld, r, 1, n);
+  issue_step(ld, r, -DEPTH, n, 0, 1, 0);
+  issue_step(ld, r, 1 - DEPTH, n, 0, 1, 1);
 }
 
 template <int DEPTH>
@@ -386,26 +429,15 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc.v[a][b][r] = 0.0f;
 
-  // Loads a step issues, in this order: [scale loads] [routed-row pair, even steps: X_LOADS]
-  // [weight slot: W_LOADS].  Step t needs slot t+1 in LDS.  Its weight rows were issued in step
-  // t+1-DEPTH; its routed rows in the even step t-DEPTH or t+1-DEPTH, in front of that step's
-  // weight rows.  So everything issued in steps t+2-DEPTH .. t-1 may still be outstanding.
-  auto issued_in = [&](int u) {  // tile loads step u issued (u < 0: the prologue plays steps -DEPTH .. -1)
-    const int s = u + DEPTH;     // slot whose weight rows step u issues
-    return (s < n ? W_LOADS : 0) + ((u & 1) == 0 && s < n ? X_LOADS : 0);
-  };
-  constexpr int STEADY = (DEPTH - 2) * W_LOADS + (DEPTH - 2) / 2 * X_LOADS;  // DEPTH is even
-  static_assert(DEPTH % 2 == 0, "routed-row pairs are issued on even steps");
+  static_assert(DEPTH % 2 == 0, "routed-row pairs start on even steps");
+  // steady state, every step issuing: what may be outstanding when step t waits for slot t+1
+  constexpr int STEADY_EVEN = DEPTH >= 4 ? (DEPTH - 2) * (W_LOADS + X_LOADS / 2) : 0;            // t even
+  constexpr int STEADY_ODD = DEPTH >= 4 ? STEADY_EVEN - X_LOADS / 2 : 0;                         // t odd
 
-  // ---- rest of the prologue (slots 0 and 1 were issued by `prefetch`), then slot 0's operands
+  // ---- rest of the prologue (steps -DEPTH and 1-DEPTH were issued by `prefetch`), then slot 0's operands
 #pragma unroll
-  for (int s2 = 2; s2 < DEPTH; ++s2) issue_prologue_step(ld, r, s2, n);
-  {  // slot 0: younger loads are those of prologue steps 1-DEPTH .. -1
-    int younger = 0;
-#pragma unroll
-    for (int u = 1 - DEPTH; u < 0; ++u) younger += issued_in(u);
-    wait_loads_and_reads_dyn(younger);
-  }
+  for (int u = 2 - DEPTH; u < 0; ++u) issue_step(ld, r, u, n, (u + DEPTH) & ~1, ((u + DEPTH) & ~1) + 1, u + DEPTH);
+  wait_loads_and_reads_dyn(loads_younger_than_slot<DEPTH>(0, -1, n));
   wg_barrier();
   Operands even, odd;
   int sx[XFRAGS], sw[WFRAGS], sxn[XFRAGS], swn[WFRAGS];
@@ -435,10 +467,12 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       Operands& cur = ODD ? odd : even;
       Operands& next = ODD ? even : odd;
       __builtin_amdgcn_sched_barrier(0);  // nothing of the previous step sinks below, nothing of this one rises above
-      wait_loads_and_reads<STEADY>();
+      wait_loads_and_reads<ODD ? STEADY_ODD : STEADY_EVEN>();
       wg_barrier();
-      // slot j+S's buffers are free; so is the routed-row buffer before it (freed a step ago)
-      const int xprev = xnext(xb, XDEPTH - 1), xcur = xb;
+      // slot j+S's buffers are free; so is the routed-row buffer before it (freed a step ago): they take
+      // the pair of routed-row slots that starts DEPTH slots ahead of this (even) or the previous (odd) step
+      const int xb0 = ODD ? xnext(xb, XDEPTH - 2) : xnext(xb, XDEPTH - 1);
+      const int xb1 = ODD ? xnext(xb, XDEPTH - 1) : xb;
       xb = xnext(xb, 1);
       const unsigned char* xnew = r.x(xb);
       const unsigned char* wnew = r.w((S + 1) % DEPTH);
@@ -461,8 +495,14 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
         // next pair's scale dwords: read here, shifted into place three MFMAs later, when they have arrived
         if constexpr (ODD && I == 11) read_scales<(S + 1) & 7, false>(sxn, swn, r.wscale(), r.xscale(), j + S + 1, xscoff, wscoff, half);
         if constexpr (ODD && I == 14) shift_scales(sxn, swn, half);
-        if constexpr (!ODD) issue_one<false, (S + DEPTH) & 7, I>(ld, r, j + S + DEPTH, S % DEPTH, xprev, xcur);
-        if constexpr (ODD && I % 4 == 1) issue_one<true, (S + DEPTH) & 7, I / 4>(ld, r, j + S + DEPTH, S % DEPTH, xprev, xcur);
+        // this step's loads: 10 on even steps (at the MFMAs that also carry reads), 8 on odd ones
+        if constexpr (DEPTH >= 4) {
+          constexpr int LE = I == 0 ? 0 : I == 1 ? 1 : I == 3 ? 2 : I == 4 ? 3 : I == 6 ? 4 : I == 7 ? 5 : I == 9 ? 6 : I == 10 ? 7 : I == 12 ? 8 : I == 13 ? 9 : -1;
+          if constexpr (!ODD && LE >= 0) issue_one<false, (S + DEPTH) & 7, LE>(ld, r, j + S + DEPTH, S % DEPTH, xb0, xb1);
+          if constexpr (ODD && I % 2 == 1) issue_one<true, (S + DEPTH) & 7, I / 2>(ld, r, j + S + DEPTH, S % DEPTH, xb0, xb1);
+        } else if constexpr (I == 8) {
+          issue_step(ld, r, j + S, n, xb0, xb1, S % DEPTH);
+        }
         __builtin_amdgcn_sched_barrier(0);
       };
       place(std::integral_constant<int, 0>{});
@@ -504,15 +544,10 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   // nobody uses), which keeps control flow out of the accumulator's live range.
   int wb = 0;  // weight buffer of slot j (j is a multiple of 8 here)
   auto advance = [&](int t_, Operands& next) {
-    int younger = 0;
-#pragma unroll
-    for (int u = 2 - DEPTH; u < 0; ++u) younger += issued_in(t_ + u);
-    wait_loads_and_reads_dyn(younger);
+    wait_loads_and_reads_dyn(loads_younger_than_slot<DEPTH>(t_ + 1, t_ - 1, n));
     wg_barrier();
-    if (t_ + DEPTH < n) {
-      if ((t_ & 1) == 0) issue_x_pair(ld, r, t_ + DEPTH, xnext(xb, XDEPTH - 1), xb);
-      issue_w(ld, r, t_ + DEPTH, wb);
-    }
+    const bool odd_step = t_ & 1;
+    issue_step(ld, r, t_, n, odd_step ? xnext(xb, XDEPTH - 2) : xnext(xb, XDEPTH - 1), odd_step ? xnext(xb, XDEPTH - 1) : xb, wb);
     xb = xnext(xb, 1);
     wb = wb + 1 == DEPTH ? 0 : wb + 1;
     read_operands(next, r.x(xb), r.w(wb), xoff, woff);
