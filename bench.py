@@ -31,7 +31,7 @@ FLOPS_TOTAL = FLOPS_GATE_UP + FLOPS_DOWN
 PEAK_FP8_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
 # HBM-side bytes of one gate/up launch: FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this script, each
 # scaled by what the same counter reads for a 1 GiB device copy (--copy-calibration): 2.0 and 1.0 KiB per unit.
-TRAFFIC_GATE_UP_BYTES = 1.127e9
+TRAFFIC_GATE_UP_BYTES = 1.105e9
 
 
 def make_inputs(dev, seed=0):

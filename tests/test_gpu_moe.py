@@ -136,6 +136,25 @@ def test_device_quantiser_is_bit_exact():
     assert np.array_equal(q[:, :2880].cpu().numpy(), mxfp8.mx_quantize(x.numpy())[0]) and not q[:, 2880:].any()
 
 
+def test_weight_layout_conversions_are_pure_permutations():
+    """K-tiled codes [E, K/64, N, 64] and slot-major scales [E, K/128, N, 4] against numpy reshapes."""
+    from pipelink_amd.host.mok import scale_pitch, weight_codes_to_k64_tiled, weight_scales_to_slot_major
+
+    g = torch.Generator().manual_seed(1)
+    e, n, k, ld = 3, 96, 320, 384
+    q = torch.randint(0, 256, (e, n, ld), dtype=torch.uint8, generator=g)
+    tiled = weight_codes_to_k64_tiled(q.cuda(), k).cpu().numpy()
+    want = q.numpy()[:, :, :k].reshape(e, n, k // 64, 64).transpose(0, 2, 1, 3)
+    assert tiled.shape == (e, k // 64, n, 64) and np.array_equal(tiled, want)
+    lds = scale_pitch(k)
+    sc = torch.randint(0, 255, (e, n, lds), dtype=torch.uint8, generator=g)
+    slot = weight_scales_to_slot_major(sc.cuda(), k).cpu().numpy()
+    nb = k // 32                                   # 10 blocks: the third slot's dword is half padding
+    padded = np.zeros((e, n, 12), dtype=np.uint8)
+    padded[:, :, :nb] = sc.numpy()[:, :, :nb]
+    assert slot.shape == (e, 3, n, 4) and np.array_equal(slot, padded.reshape(e, n, 3, 4).transpose(0, 2, 1, 3))
+
+
 def test_argument_errors_are_reported_not_launched(cell):
     from pipelink_amd.host import mok_inputs
     from pipelink_amd.host.backend import PlkError
