@@ -17,6 +17,8 @@
 extern "C" {
 #endif
 
+#ifndef PLK_STATUS_CODES_DEFINED
+#define PLK_STATUS_CODES_DEFINED
 enum {
   PLK_OK = 0,
   PLK_E_VERSION = 1,
@@ -27,6 +29,7 @@ enum {
   PLK_E_BUILD = 6,
   PLK_E_RELEASE = 7
 };
+#endif
 
 typedef struct plk_hip_module plk_hip_module;     /* one loaded code object */
 typedef struct plk_hip_function plk_hip_function; /* one kernel of it */

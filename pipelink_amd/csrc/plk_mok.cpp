@@ -8,19 +8,14 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <string>
 #include <vector>
 
-#include "../stages/mok/include/mok_abi.h"
+#include "plk_mok_residues.hpp"
 
 extern "C" int plk_hip_set_error(int code, const char* what);
 
-namespace {
-constexpr int TILE_X = 256;  // routed rows per workgroup tile   (fact mok.gemm.TILE_X)
-constexpr int TILE_W = 256;  // weight rows per workgroup tile   (fact mok.gemm.TILE_W)
-constexpr int K_STEP = 64;
-constexpr int MAX_EXPERTS = 256;
-constexpr int NUM_XCD = 8;
-}  // namespace
+using plk_mok::NUM_XCD;
 
 struct plk_mok_session {
   plk_hip_module* module = nullptr;
@@ -31,46 +26,37 @@ struct plk_mok_session {
   int32_t compute_units = 0;
 };
 
+static plk_mok::Dims dims_of(const plk_mok_problem* p, int pass) {
+  plk_mok::Dims d;
+  d.tokens = p->num_tokens;
+  d.hidden = p->hidden;
+  d.intermediate = p->intermediate;
+  d.experts = p->num_experts;
+  d.routed_rows = p->routed_rows;
+  d.ld_q_h = p->ld_q_h ? p->ld_q_h : p->hidden;
+  d.ld_q_i = p->ld_q_i ? p->ld_q_i : p->intermediate;
+  d.ld_sc_h = p->ld_sc_h;
+  d.ld_sc_i = p->ld_sc_i;
+  d.pass = pass;
+  d.swiglu_limit = p->swiglu_limit;
+  return d;
+}
+
 static int check_problem(const plk_mok_problem* p) {
   if (!p || p->struct_bytes != sizeof(plk_mok_problem))
     return plk_hip_set_error(PLK_E_VERSION, "plk_mok: problem struct size mismatch");
-  if (p->num_experts <= 0 || p->num_experts > MAX_EXPERTS)
-    return plk_hip_set_error(PLK_E_CAPACITY, "plk_mok: num_experts must be in 1..256");
-  if (p->hidden <= 0 || p->intermediate <= 0 || p->hidden % K_STEP || p->intermediate % K_STEP)
-    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: hidden and intermediate must be positive multiples of 64");
-  if (p->ld_sc_h % 16 || p->ld_sc_i % 16 || p->ld_sc_h * 32 < p->hidden || p->ld_sc_i * 32 < p->intermediate)
-    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: scale pitch must be a multiple of 16 covering K/32 blocks");
-  if ((p->ld_q_h && (p->ld_q_h < p->hidden || p->ld_q_h % 16)) || (p->ld_q_i && (p->ld_q_i < p->intermediate || p->ld_q_i % 16)))
-    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: code row pitch must be a multiple of 16 and at least K");
-  if (p->num_tokens < 0 || p->routed_rows < 0)
-    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: negative row count");
-  {
-    // the kernel addresses one operand with 32-bit byte offsets from its base
-    const int64_t ldh = p->ld_q_h ? p->ld_q_h : p->hidden, ldi = p->ld_q_i ? p->ld_q_i : p->intermediate;
-    const int64_t lim = (int64_t)1 << 32;
-    if (p->num_tokens * ldh >= lim || p->routed_rows * ldi >= lim || (int64_t)p->intermediate * p->hidden >= lim)
-      return plk_hip_set_error(PLK_E_CAPACITY, "plk_mok: an operand (rows x row pitch) must stay below 4 GiB");
+  const plk_mok::Dims d = dims_of(p, 1);
+  if (const char* what = plk_mok::check_dims(d)) {
+    static thread_local std::string msg;
+    msg = std::string("plk_mok: ") + what;
+    const bool capacity = d.experts <= 0 || d.experts > plk_mok::MAX_EXPERTS || msg.find("4 GiB") != std::string::npos;
+    return plk_hip_set_error(capacity ? PLK_E_CAPACITY : PLK_E_ARGUMENT, msg.c_str());
   }
   if (p->routed_rows && (!p->x_q || !p->x_sc || !p->tokens_per_expert || !p->w_gate_q || !p->w_gate_sc ||
                          !p->w_up_q || !p->w_up_sc || !p->w_down_q || !p->w_down_sc || !p->hidden_q ||
                          !p->hidden_sc || !p->y))
     return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok: null device address");
   return PLK_OK;
-}
-
-// activations: row-major codes with pitch ld_q, row-major scales with pitch ld_sc;
-// weights (per_expert): K-tiled codes [K/64, rows, 64], slot-major scales [K/128, rows, 4]
-static MokMxView view(uint64_t q, uint64_t sc, int64_t rows, int k, int ld_q, int ld_sc, bool per_expert) {
-  MokMxView v{};
-  v.q = (const uint8_t*)(uintptr_t)q;
-  v.sc = (const uint8_t*)(uintptr_t)sc;
-  v.rows = (int32_t)rows;
-  v.k = k;
-  v.ld_q = per_expert ? 64 : ld_q;
-  v.ld_sc = ld_sc;
-  v.expert_pitch_q = per_expert ? rows * (int64_t)k : 0;
-  v.expert_pitch_sc = per_expert ? (int64_t)((k + 127) / 128) * rows * 4 : 0;
-  return v;
 }
 
 extern "C" {
@@ -127,32 +113,12 @@ int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass,
   if (rc != PLK_OK) return rc;
   if (p->routed_rows == 0) return PLK_OK;  // nothing routed to this rank
 
-  const int H = p->hidden, I = p->intermediate, E = p->num_experts;
-  MokFrameworkParams fw{};
-  fw.tokens_per_expert = (const int32_t*)(uintptr_t)p->tokens_per_expert;
-  fw.num_experts = E;
-  fw.op = pass == 1 ? MOK_GEMM_FWD_ROUTED_GATE_UP : MOK_GEMM_FWD_ROUTED_DOWN;
-  fw.num_col_tiles = pass == 1 ? (I + TILE_W / 2 - 1) / (TILE_W / 2) : (H + TILE_W - 1) / TILE_W;
-
-  MokGemmResidue g{};
-  const int ldh = p->ld_q_h ? p->ld_q_h : H, ldi = p->ld_q_i ? p->ld_q_i : I;
-  g.x = view(p->x_q, p->x_sc, p->num_tokens, H, ldh, p->ld_sc_h, false);
-  g.hidden = view(p->hidden_q, p->hidden_sc, p->routed_rows, I, ldi, p->ld_sc_i, false);
-  g.w_gate = view(p->w_gate_q, p->w_gate_sc, I, H, ldh, p->ld_sc_h, true);
-  g.w_up = view(p->w_up_q, p->w_up_sc, I, H, ldh, p->ld_sc_h, true);
-  g.w_down = view(p->w_down_q, p->w_down_sc, H, I, ldi, p->ld_sc_i, true);
-  g.row_token = (const int32_t*)(uintptr_t)p->row_token;
-  g.y = (uint16_t*)(uintptr_t)p->y;
-  g.ld_y = H;
-
-  MokActResidue a{};
-  a.hidden_q = (uint8_t*)(uintptr_t)p->hidden_q;
-  a.hidden_sc = (uint8_t*)(uintptr_t)p->hidden_sc;
-  a.rows = p->routed_rows;
-  a.cols = I;
-  a.ld_q = ldi;
-  a.ld_sc = p->ld_sc_i;
-  a.swiglu_limit = p->swiglu_limit;
+  const plk_mok::Dims d = dims_of(p, pass);
+  const MokFrameworkParams fw = plk_mok::framework_params(d, p->tokens_per_expert);
+  const MokGemmResidue g = plk_mok::gemm_residue(
+      d, plk_mok::GemmAddresses{p->x_q, p->x_sc, p->w_gate_q, p->w_gate_sc, p->w_up_q, p->w_up_sc, p->w_down_q, p->w_down_sc,
+                                p->hidden_q, p->hidden_sc, p->y, p->row_token});
+  const MokActResidue a = plk_mok::act_residue(d, p->hidden_q, p->hidden_sc);
 
   const int slot = pass - 1;
   std::vector<unsigned char> image(s->link.params_bytes, 0);
@@ -167,8 +133,7 @@ int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass,
 
   // persistent grid: the solved occupancy on every CU, a multiple of the XCD count, but no
   // more workgroups than there can be tiles
-  const int64_t max_row_tiles = (p->routed_rows + TILE_X - 1) / TILE_X + E;
-  const int64_t max_tiles = max_row_tiles * fw.num_col_tiles;
+  const int64_t max_tiles = plk_mok::max_workgroups(d);
   int64_t wgs = (int64_t)s->compute_units * s->link.workgroups_per_cu;
   if (wgs > max_tiles) wgs = max_tiles;
   wgs = (wgs + NUM_XCD - 1) / NUM_XCD * NUM_XCD;

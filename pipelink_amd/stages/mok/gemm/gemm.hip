@@ -467,8 +467,7 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       Operands& cur = ODD ? odd : even;
       Operands& next = ODD ? even : odd;
       __builtin_amdgcn_sched_barrier(0);  // nothing of the previous step sinks below, nothing of this one rises above
-      wait_loads_and_reads<ODD ? STEADY_ODD : STEADY_EVEN>();
-      wg_barrier();
+      // (the wait and the barrier that free slot j+S's buffers sit behind the step's second MFMA, see below:)
       // slot j+S's buffers are free; so is the routed-row buffer before it (freed a step ago): they take
       // the pair of routed-row slots that starts DEPTH slots ahead of this (even) or the previous (odd) step
       const int xb0 = ODD ? xnext(xb, XDEPTH - 2) : xnext(xb, XDEPTH - 1);
@@ -476,30 +475,38 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       xb = xnext(xb, 1);
       const unsigned char* xnew = r.x(xb);
       const unsigned char* wnew = r.w((S + 1) % DEPTH);
-      // The step, MFMA by MFMA.  One LDS unit and one texture-address unit serve the four
-      // waves: an LDS read costs the unit about 8 cycles and a 1 KB load about 16, so a wave
+      // The step, MFMA by MFMA.  The first two MFMAs only need registers; the wait and the
+      // barrier come behind them, so the matrix pipe has 128 cycles of work while the waves
+      // meet.  After the barrier: one LDS unit and one texture-address unit serve the four
+      // waves, an LDS read costs the unit about 8 cycles and a 1 KB load about 16, so a wave
       // puts at most two reads and one load between two 64-cycle MFMAs, or the MFMA behind
-      // them issues late.  The reads sit in the first 12 of the 16 places (the barrier of the
-      // next step wants them back), the loads are spread over all of them.  The scheduler may
-      // not move anything from one place to another.
+      // them issues late.  The reads sit in places 2..12 of 16 (the next barrier wants them
+      // back), the loads are spread over 2..15.  The scheduler may not move anything from one
+      // place to another.
       auto place = [&](auto I_) {
         constexpr int I = decltype(I_)::value;
         constexpr int A = I / XFRAGS, B = I % XFRAGS;
         acc.v[A][B] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cur.w[A], cur.x[B], acc.v[A][B], 0, 0, ODD ? 2 : 0,
                                                                       sw[A], ODD ? 2 : 0, sx[B]);
         __builtin_amdgcn_sched_barrier(0);  // the MFMA goes first: the pipe is what must not wait
+        if constexpr (I == 1) {
+          wait_loads_and_reads<ODD ? STEADY_ODD : STEADY_EVEN>();
+          wg_barrier();
+          __builtin_amdgcn_sched_barrier(0);
+        }
         // operand fragment K of the next slot: routed rows first, they are needed by the first MFMAs
-        constexpr int K = I == 0 ? 0 : I == 1 ? 1 : I == 3 ? 2 : I == 4 ? 3 : I == 6 ? 4 : I == 7 ? 5 : I == 9 ? 6 : I == 10 ? 7 : -1;
+        constexpr int K = I == 2 ? 0 : I == 3 ? 1 : I == 5 ? 2 : I == 6 ? 3 : I == 8 ? 4 : I == 9 ? 5 : I == 11 ? 6 : I == 12 ? 7 : -1;
         if constexpr (K >= 0 && K < XFRAGS) next.x[K] = read_frag(xnew, xoff[K]);
         if constexpr (K >= XFRAGS) next.w[K - XFRAGS] = read_frag(wnew, woff[K - XFRAGS]);
-        // next pair's scale dwords: read here, shifted into place three MFMAs later, when they have arrived
-        if constexpr (ODD && I == 11) read_scales<(S + 1) & 7, false>(sxn, swn, r.wscale(), r.xscale(), j + S + 1, xscoff, wscoff, half);
-        if constexpr (ODD && I == 14) shift_scales(sxn, swn, half);
-        // this step's loads: 10 on even steps (at the MFMAs that also carry reads), 8 on odd ones
+        // next pair's scale dwords: read here, shifted into place two MFMAs later, when they have arrived
+        if constexpr (ODD && I == 13) read_scales<(S + 1) & 7, false>(sxn, swn, r.wscale(), r.xscale(), j + S + 1, xscoff, wscoff, half);
+        if constexpr (ODD && I == 15) shift_scales(sxn, swn, half);
+        // this step's loads: 10 on even steps, 8 on odd ones
         if constexpr (DEPTH >= 4) {
-          constexpr int LE = I == 0 ? 0 : I == 1 ? 1 : I == 3 ? 2 : I == 4 ? 3 : I == 6 ? 4 : I == 7 ? 5 : I == 9 ? 6 : I == 10 ? 7 : I == 12 ? 8 : I == 13 ? 9 : -1;
+          constexpr int LE = I == 2 ? 0 : I == 3 ? 1 : I == 5 ? 2 : I == 6 ? 3 : I == 8 ? 4 : I == 9 ? 5 : I == 11 ? 6 : I == 12 ? 7 : I == 14 ? 8 : I == 15 ? 9 : -1;
+          constexpr int LO = (I >= 2 && I % 2 == 0) ? (I - 2) / 2 : I == 15 ? 7 : -1;
           if constexpr (!ODD && LE >= 0) issue_one<false, (S + DEPTH) & 7, LE>(ld, r, j + S + DEPTH, S % DEPTH, xb0, xb1);
-          if constexpr (ODD && I % 2 == 1) issue_one<true, (S + DEPTH) & 7, I / 2>(ld, r, j + S + DEPTH, S % DEPTH, xb0, xb1);
+          if constexpr (ODD && LO >= 0) issue_one<true, (S + DEPTH) & 7, LO>(ld, r, j + S + DEPTH, S % DEPTH, xb0, xb1);
         } else if constexpr (I == 8) {
           issue_step(ld, r, j + S, n, xb0, xb1, S % DEPTH);
         }

@@ -32,6 +32,16 @@ def test_every_declared_symbol_is_exported(lib):
     assert not missing, missing
 
 
+def test_every_provider_entry_point_is_exported(lib):
+    """include/plk_host_abi_v2.h declares abi / query / build / release once per owner suffix."""
+    text = open(os.path.join(ROOT, "include", "plk_host_abi_v2.h")).read()
+    suffixes = re.findall(r"^PLK_DECLARE_OWNER\((\w+)\)", text, flags=re.M)
+    assert suffixes == ["mok_gemm", "mok_act", "mok_framework"]
+    missing = [f"pipelink_params_{verb}_{s}" for s in suffixes for verb in ("abi", "query", "build", "release")
+               if not hasattr(lib, f"pipelink_params_{verb}_{s}")]
+    assert not missing, missing
+
+
 def test_python_binding_covers_the_headers():
     from pipelink_amd.host.backend import SIGNATURES, load_library
 

@@ -155,6 +155,46 @@ def test_weight_layout_conversions_are_pure_permutations():
     assert slot.shape == (e, 3, n, 4) and np.array_equal(slot, padded.reshape(e, n, 3, 4).transpose(0, 2, 1, 3))
 
 
+def test_broker_route_gives_the_same_bytes_as_the_forward_entry(cell):
+    """open_host (providers' abi / query / build -> params image -> launch) against plk_mok_forward."""
+    import json
+    from pipelink_amd.host import broker, mok_inputs
+    from pipelink_amd.host.backend import HipBackend
+    from pipelink_amd.host.mok import scale_pitch, weight_codes_to_k64_tiled, weight_scales_to_slot_major
+    from pipelink_amd.stages.mok import build as mok_build
+
+    T, H, I, E, k = 300, 320, 192, 4, 2
+    inp = mok_inputs.generate(T, H, I, E, k, seed=1)
+    want = _run(cell[0], inp, H, I)
+    dev = torch.device("cuda:0")
+    d = {n: v.to(dev) for n, v in inp.__dict__.items()}
+    t = dict(x_q=d["x_q"], x_sc=d["x_sc"], row_token=d["row_token"], tokens_per_expert=d["tokens_per_expert"],
+             w_gate_q=weight_codes_to_k64_tiled(d["w_gate_q"], H), w_gate_sc=weight_scales_to_slot_major(d["w_gate_sc"], H),
+             w_up_q=weight_codes_to_k64_tiled(d["w_up_q"], H), w_up_sc=weight_scales_to_slot_major(d["w_up_sc"], H),
+             w_down_q=weight_codes_to_k64_tiled(d["w_down_q"], I), w_down_sc=weight_scales_to_slot_major(d["w_down_sc"], I))
+    rows = int(inp.tokens_per_expert.sum())
+    t["hidden_q"] = torch.full((rows, I), 0xFF, dtype=torch.uint8, device=dev)
+    t["hidden_sc"] = torch.full((rows, scale_pitch(I)), 0xFF, dtype=torch.uint8, device=dev)
+    t["y"] = torch.full((rows, H), float("nan"), dtype=torch.bfloat16, device=dev)
+    res = lambda n: broker.Resource(t[n].data_ptr(), t[n].numel() * t[n].element_size())
+    resources = {"mok.framework": {"tokens_per_expert": res("tokens_per_expert")},
+                 "mok.gemm": {n: res(n) for n in ("x_q", "x_sc", "w_gate_q", "w_gate_sc", "w_up_q", "w_up_sc", "w_down_q",
+                                                  "w_down_sc", "hidden_q", "hidden_sc", "y", "row_token")},
+                 "mok.act": {"hidden_q": res("hidden_q"), "hidden_sc": res("hidden_sc")}}
+    scalars = {"mok.num_local_tokens": T, "mok.hidden": H, "mok.intermediate": I, "mok.num_local_experts": E,
+               "mok.swiglu_limit": 7.0, "mok.pass": 1, "mok.precision": 1, "mok.routed_rows": rows, "mok.ld_q_h": H,
+               "mok.ld_q_i": I, "mok.ld_sc_h": scale_pitch(H), "mok.ld_sc_i": scale_pitch(I)}
+    paths = mok_build.images()
+    link = json.loads(paths["link_json"].read_text())
+    be = HipBackend(0, torch.cuda.current_stream().cuda_stream)
+    for pass_ in (1, 2):
+        with broker.open_host(link, paths["linked"].read_bytes(), resources, dict(scalars, **{"mok.pass": pass_}), be) as s:
+            s.launch()
+            be.synchronize()
+    assert np.array_equal(t["hidden_q"].cpu().numpy(), want[0]) and np.array_equal(t["hidden_sc"].cpu().numpy(), want[1])
+    assert torch.equal(t["y"].cpu().view(torch.int16), want[2].view(torch.int16))
+
+
 def test_argument_errors_are_reported_not_launched(cell):
     from pipelink_amd.host import mok_inputs
     from pipelink_amd.host.backend import PlkError

@@ -1,0 +1,137 @@
+"""Host ABI v2: the providers' abi / query / build / release against the broker's mirrors, without a GPU.
+
+Pins (reference: pipec/src/pipec2/host/include/pipelink_host_abi_v2.h:21-28,43-47,293-300 and
+campaigns/mok/port/gemm/provider.cu:217-303): version and struct_bytes checks, status codes,
+capacity rules, caller-owned residue bytes, null-session release, and that the params image the
+broker assembles through the providers is byte-identical to the one the forward entry builds."""
+import ctypes
+import json
+import os
+from ctypes import byref, sizeof
+
+import pytest
+
+from pipelink_amd.host import broker
+from pipelink_amd.host.backend import PlkError, load_library
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+SCALARS = {"mok.num_local_tokens": 512, "mok.hidden": 320, "mok.intermediate": 192, "mok.num_local_experts": 4,
+           "mok.swiglu_limit": 7.0, "mok.pass": 1, "mok.precision": 1, "mok.routed_rows": 1024, "mok.ld_q_h": 384,
+           "mok.ld_q_i": 256, "mok.ld_sc_h": 16, "mok.ld_sc_i": 16}
+LINK = {"threads": 256, "dyn_smem_bytes": 161800, "kernel_symbol": "pipelink_kernel", "workgroups_per_cu": 1,
+        "params": {"total_bytes": 344, "entries": [{"stage_id": "mok.framework", "offset": 0, "bytes": 40},
+                                                   {"stage_id": "mok.gemm", "offset": 40, "bytes": 264},
+                                                   {"stage_id": "mok.act", "offset": 304, "bytes": 40}]}}
+
+
+def _resources(scalars=SCALARS, row_token=True):
+    """Fake device addresses (nothing is dereferenced on the host): 1 MiB apart, 256-byte aligned."""
+    out, addr = {}, 0x7F0000000000
+    for stage, chans in broker._shapes(scalars).items():
+        out[stage] = {}
+        for name, (bits, _, extents) in chans.items():
+            if name == "row_token" and not row_token:
+                continue
+            size = bits // 8
+            for e in extents:
+                size *= e
+            out[stage][name] = broker.Resource(addr, size)
+            addr += 1 << 24
+    return out
+
+
+def test_abi_report_matches_the_ctypes_mirrors():
+    lib = load_library()
+    for stage in broker.OWNERS:
+        rep = broker.Owner(lib, stage).report()          # raises on any size / alignment / digest mismatch
+        assert rep.entry_count == 20 + len(broker.OWNERS[stage][1])
+    assert sizeof(broker.MokGemmResidue) == 264 and sizeof(broker.MokActResidue) == 40 and sizeof(broker.MokFrameworkParams) == 40
+
+
+def test_abi_report_rejects_wrong_version_capacity_and_ids():
+    lib = load_library()
+    owner = broker.Owner(lib, "mok.gemm")
+    rep = broker.AbiReport()
+    rep.header = broker.Header(3, sizeof(rep))
+    assert owner.abi(byref(rep)) == 1                     # PLK_E_VERSION
+    rep.header = broker.Header(2, sizeof(rep) - 8)
+    assert owner.abi(byref(rep)) == 1
+    rep.header = broker.Header(2, sizeof(rep))
+    entries = (broker.LayoutEntry * 22)()
+    rep.entries, rep.entry_capacity = entries, 21
+    assert owner.abi(byref(rep)) == 2                     # PLK_E_CAPACITY
+    rep.entry_capacity = 22
+    assert owner.abi(byref(rep)) == 4                     # PLK_E_CONTRACT: ids not pre-filled
+
+
+def test_plan_builds_the_same_image_as_the_structs_say():
+    res = _resources()
+    image, geometry, owners = broker.plan(LINK, res, SCALARS, compute_units=256)
+    assert len(image) == 344 and geometry["block"] == (256, 1, 1) and geometry["dyn_lds"] == 161800
+    assert geometry["grid"][0] % 8 == 0 and 0 < geometry["grid"][0] <= 256
+    fw = broker.MokFrameworkParams.from_buffer_copy(image[0:40])
+    g = broker.MokGemmResidue.from_buffer_copy(image[40:304])
+    a = broker.MokActResidue.from_buffer_copy(image[304:344])
+    assert fw.tokens_per_expert == res["mok.framework"]["tokens_per_expert"].address
+    assert (fw.num_experts, fw.op, fw.num_col_tiles) == (4, 3, 2)             # gate/up: ceil(192 / 128) column tiles
+    assert (g.x.q, g.x.rows, g.x.k, g.x.ld_q, g.x.ld_sc) == (res["mok.gemm"]["x_q"].address, 512, 320, 384, 16)
+    assert (g.w_gate.rows, g.w_gate.k, g.w_gate.ld_q, g.w_gate.expert_pitch_q, g.w_gate.expert_pitch_sc) == \
+        (192, 320, 64, 192 * 320, 3 * 192 * 4)
+    assert (g.w_down.rows, g.w_down.k, g.w_down.expert_pitch_q) == (320, 192, 320 * 192)
+    assert (g.hidden.rows, g.hidden.ld_q, g.y, g.ld_y) == (1024, 256, res["mok.gemm"]["y"].address, 320)
+    assert g.row_token == res["mok.gemm"]["row_token"].address
+    assert (a.rows, a.cols, a.ld_q, a.ld_sc, a.swiglu_limit) == (1024, 192, 256, 16, 7.0)
+    for o in reversed(owners):
+        assert o.release(o.session) == 0                  # null sessions release fine
+    down = dict(SCALARS, **{"mok.pass": 2})
+    image2, _, _ = broker.plan(LINK, res, down, compute_units=256)
+    fw2 = broker.MokFrameworkParams.from_buffer_copy(image2[0:40])
+    assert (fw2.op, fw2.num_col_tiles) == (5, 2) and image2[40:] == image[40:]
+
+
+def test_optional_row_token_channel_may_be_absent():
+    res = _resources(row_token=False)
+    image, _, _ = broker.plan(LINK, res, SCALARS, compute_units=256)
+    assert broker.MokGemmResidue.from_buffer_copy(image[40:304]).row_token is None
+
+
+@pytest.mark.parametrize("mutate,status", [
+    (lambda s, r, l: s.update({"mok.hidden": 96}), 3),                     # not a multiple of 64: PLK_E_ARGUMENT
+    (lambda s, r, l: s.pop("mok.routed_rows"), 3),                         # a scalar is missing
+    (lambda s, r, l: s.update({"mok.precision": 2}), 3),                   # only MXFP8 is built
+    (lambda s, r, l: l.update(threads=512), 4),                            # block shape: PLK_E_CONTRACT
+    (lambda s, r, l: r["mok.gemm"].update(y=broker.Resource(r["mok.gemm"]["y"].address, 16)), 5),   # too small
+    (lambda s, r, l: r["mok.gemm"].update(x_q=broker.Resource(r["mok.gemm"]["x_q"].address + 4,
+                                                              r["mok.gemm"]["x_q"].allocation_bytes)), 5),  # misaligned
+    (lambda s, r, l: l["params"]["entries"][1].update(bytes=128), 2),      # residue capacity: PLK_E_CAPACITY
+])
+def test_provider_and_broker_reject_bad_inputs(mutate, status):
+    scalars, res, link = dict(SCALARS), _resources(), json.loads(json.dumps(LINK))
+    mutate(scalars, res, link)
+    with pytest.raises(PlkError) as err:
+        broker.plan(link, res, scalars, compute_units=256)
+    assert err.value.status == status
+
+
+def test_build_checks_the_resource_records_itself():
+    """Call build directly with a resource smaller than the demand: PLK_E_RESOURCE, and no session."""
+    lib = load_library()
+    owner = broker.Owner(lib, "mok.act")
+    shared = broker._Scalars(SCALARS)
+    common = broker.Common()
+    common.header = broker.Header(2, sizeof(common))
+    common.channel_count, common.shared = 2, shared.pointer
+    common.block, common.cluster = broker.Dim3(256, 1, 1), broker.Dim3(1, 1, 1)
+    devres = (broker.DeviceResource * 2)(broker.DeviceResource(1, 2, 0x1000, 64, 0, 0, 0, None, 0),
+                                         broker.DeviceResource(2, 2, 0x2000, 1 << 20, 0, 0, 0, None, 0))
+    r = broker.Resources()
+    r.header = broker.Header(2, sizeof(r))
+    r.channel_count, r.channels, r.shared = 2, devres, shared.pointer
+    out = ctypes.create_string_buffer(40)
+    session = ctypes.c_void_p(123)
+    assert owner.build(byref(common), None, byref(r), out, 40, None, 0, byref(session)) == 5
+    assert session.value is None
+    assert owner.build(byref(common), None, byref(r), out, 40, None, 1, byref(session)) == 2      # transfers are not reported
+    assert owner.build(byref(common), ctypes.c_void_p(1), byref(r), out, 40, None, 0, byref(session)) == 3   # args must be null
+    assert owner.release(ctypes.c_void_p(1)) == 7 and owner.release(None) == 0
