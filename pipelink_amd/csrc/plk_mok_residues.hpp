@@ -37,9 +37,10 @@ inline const char* check_dims(const Dims& d) {
     return "code row pitch must be a multiple of 16 and at least K";
   if (d.tokens < 0 || d.routed_rows < 0) return "negative row count";
   // the kernel addresses one operand with 32-bit byte offsets from its base
-  const int64_t lim = (int64_t)1 << 32;
+  // and marks rows past the end of a tile with an offset in the last 16 MiB of that range
+  const int64_t lim = ((int64_t)1 << 32) - ((int64_t)1 << 24);
   if ((int64_t)d.tokens * d.ld_q_h >= lim || (int64_t)d.routed_rows * d.ld_q_i >= lim || (int64_t)d.intermediate * d.hidden >= lim)
-    return "an operand (rows x row pitch) must stay below 4 GiB";
+    return "an operand (rows x row pitch) must stay 16 MiB below 4 GiB";
   return nullptr;
 }
 

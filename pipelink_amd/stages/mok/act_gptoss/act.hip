@@ -29,10 +29,18 @@ constexpr int STAGE_SCALE_OFF = TILE_X * STAGE_PITCH;   // [row][4] scale bytes 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
+// v_min_f32 as written: fminf() first quiets a signalling NaN with an extra instruction per
+// element, which an MFMA accumulator cannot hold
+__device__ __forceinline__ float min_raw(float a, float b) {
+  float r;
+  asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
 template <bool CLAMPED>
 __device__ __forceinline__ float swiglu(float gate, float up, float limit) {
   if (CLAMPED) {
-    gate = fminf(gate, limit);
+    gate = min_raw(gate, limit);
     up = __builtin_amdgcn_fmed3f(up, -limit, limit);
   }
   // (up + 1) * gate * sigmoid(alpha * gate) with the hardware exp2 and reciprocal, as in the
@@ -41,20 +49,22 @@ __device__ __forceinline__ float swiglu(float gate, float up, float limit) {
   return (up + 1.0f) * (gate * __builtin_amdgcn_rcpf(den));
 }
 
-// round two floats to bf16 (nearest even, v_cvt_pk_bf16_f32) and widen them back
-__device__ __forceinline__ void bf16_round2(float& a, float& b) {
-  const f32x2 v = {a, b};
-  const uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
-  a = __uint_as_float(bits << 16);
-  b = __uint_as_float(bits & 0xFFFF0000u);
-}
+typedef short s16x2 __attribute__((ext_vector_type(2)));
 
-// e4m3 (OCP) pack of four floats already scaled into [-448, 448]
-__device__ __forceinline__ uint32_t pack_e4m3x4(float a, float b, float c, float d) {
-  int v = 0;
-  v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, v, false);
-  v = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
-  return (uint32_t)v;
+// Four floats -> four e4m3 codes of a block whose scale is `scale` (a power of two): round to
+// bf16 (nearest even, v_cvt_pk_bf16_f32: the reference rounds to bf16 before quantising,
+// swiglu.cuh:175), divide by the scale and round to e4m3 (v_cvt_scalef32_pk_fp8_bf16, nearest
+// even, exact division).  That conversion does not saturate (a quotient above 448 becomes NaN),
+// so the floats are first clamped to +-448 * scale; the bound is a bf16 number, so clamping
+// before the bf16 rounding gives what clamping after it would (measured against the separate
+// multiply / clamp / v_cvt_pk_fp8_f32 sequence over a sweep of mantissas, exponents and scales).
+__device__ __forceinline__ uint32_t quantise4(float a, float b, float c, float d, float limit, float scale) {
+  const f32x2 lo = {__builtin_amdgcn_fmed3f(a, -limit, limit), __builtin_amdgcn_fmed3f(b, -limit, limit)};
+  const f32x2 hi = {__builtin_amdgcn_fmed3f(c, -limit, limit), __builtin_amdgcn_fmed3f(d, -limit, limit)};
+  s16x2 v = {0, 0};
+  v = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(v, __builtin_convertvector(lo, bf16x2), scale, false);
+  v = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(v, __builtin_convertvector(hi, bf16x2), scale, true);
+  return __builtin_bit_cast(uint32_t, v);
 }
 
 template <bool CLAMPED>
@@ -77,22 +87,24 @@ __device__ __forceinline__ void forward(const MokActResidue& p, const MokActTask
       for (int r = 0; r < 16; r += 2) {
         h[r] = swiglu<CLAMPED>(acc.v[a][b][r], acc.v[a + 2][b][r], p.swiglu_limit);
         h[r + 1] = swiglu<CLAMPED>(acc.v[a][b][r + 1], acc.v[a + 2][b][r + 1], p.swiglu_limit);
-        bf16_round2(h[r], h[r + 1]);  // the reference rounds to bf16 before quantising (swiglu.cuh:175)
-        amax = fmaxf(amax, fmaxf(fabsf(h[r]), fabsf(h[r + 1])));
+        amax = fmaxf(fmaxf(amax, fabsf(h[r])), fabsf(h[r + 1]));
       }
       // the other 16 columns of this row's block live in lane ^ 32
       amax = fmaxf(amax, __shfl_xor(amax, 32));
-      int e = (int)((__float_as_uint(amax) >> 23) & 0xFFu) - 8;  // floor(log2(amax)) - 8 + 127
-      e = e < 0 ? 0 : e;                                          // amax < 2^-118: scale byte 0
-      const float inv = __uint_as_float((uint32_t)(254 - e) << 23);  // 2^(127 - e), e <= 247
+      // The block's scale comes from the largest bf16-rounded magnitude; rounding is monotonic,
+      // so that is the rounded largest magnitude.
+      const f32x2 am = {amax, 0.0f};
+      const uint32_t am_bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(am, bf16x2));
+      int e = (int)((am_bits >> 7) & 0xFFu) - 8;  // floor(log2(amax)) - 8 + 127
+      e = e < 0 ? 0 : e;                          // amax < 2^-118: scale byte 0
+      // 2^(e - 127), a denormal for byte 0; the conversion only looks at the exponent the byte stands for
+      const uint32_t scale_bits = (uint32_t)e << 23;
+      const float scale = __uint_as_float(scale_bits > 0x00400000u ? scale_bits : 0x00400000u);
+      const float limit = __uint_as_float(((uint32_t)(e + 8) << 23) | 0x00600000u);  // 448 * 2^(e - 127), e <= 246
       unsigned char* dst = stage + trow * STAGE_PITCH + tcol + 4 * half;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        float s[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) s[j] = __builtin_amdgcn_fmed3f(h[4 * q + j] * inv, -448.0f, 448.0f);
-        *reinterpret_cast<uint32_t*>(dst + 8 * q) = pack_e4m3x4(s[0], s[1], s[2], s[3]);
-      }
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<uint32_t*>(dst + 8 * q) = quantise4(h[4 * q], h[4 * q + 1], h[4 * q + 2], h[4 * q + 3], limit, scale);
       if (half == 0) stage[STAGE_SCALE_OFF + trow * 4 + (tcol >> 5)] = (uint8_t)e;
     }
   }

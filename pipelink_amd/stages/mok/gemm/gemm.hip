@@ -54,9 +54,16 @@ constexpr int W_LOADS = W_GROUPS;              // loads of one weight slot issue
 // Loads are buffer loads: a 128-bit resource (base address and byte extent, in scalar
 // registers), a 32-bit lane offset that is fixed for the tile, and the contraction offset as
 // the instruction's scalar offset -- no address arithmetic per load, and a read past the
-// extent returns zeros instead of faulting.  One operand of one expert is below 4 GiB (the
-// host checks).
+// extent returns zeros instead of faulting.  One operand of one expert is 16 MiB below 4 GiB
+// (the host checks).
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
+
+// Lane offset of the rows and columns a tile has past the end of its expert's rows or of the
+// weight matrix: beyond every extent (the host keeps operands 16 MiB below 4 GiB), so the
+// load brings zeros without touching memory, and the matrix pipe multiplies zeros there,
+// which costs it far less power than multiplying a copy of the last row would.  Nothing
+// depends on the zeros: those outputs are never stored.
+constexpr uint32_t PAST_THE_END = 0xFF000000u;
 
 __device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);  // raw, 32-bit data
@@ -279,16 +286,16 @@ __device__ __forceinline__ void gather_rows(const MokGemmResidue& g, const MokGe
 #pragma unroll
   for (int i = 0; i < X_GROUPS; ++i) {
     const int trow = (wave * X_GROUPS + i) * 16 + lrow;  // tile-local routed row
-    int row = t.row_begin + trow;
-    row = row < t.row_end ? row : t.row_end - 1;
-    const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
-    c.xsrc[i] = (uint32_t)src * (uint32_t)act.ld_q + chunk;
+    const int row = t.row_begin + trow;
+    const int safe = row < t.row_end ? row : t.row_end - 1;
+    const int src = (gate_up && g.row_token) ? g.row_token[safe] : safe;
+    c.xsrc[i] = row < t.row_end ? (uint32_t)src * (uint32_t)act.ld_q + chunk : PAST_THE_END;
   }
   // routed-row scales: thread tid fetches row tid's 16-byte piece
-  int row = t.row_begin + tid;
-  row = row < t.row_end ? row : t.row_end - 1;
-  const int src = (gate_up && g.row_token) ? g.row_token[row] : row;
-  c.xscsrc = (uint32_t)src * (uint32_t)act.ld_sc;
+  const int row = t.row_begin + tid;
+  const int safe = row < t.row_end ? row : t.row_end - 1;
+  const int src = (gate_up && g.row_token) ? g.row_token[safe] : safe;
+  c.xscsrc = row < t.row_end ? (uint32_t)src * (uint32_t)act.ld_sc : PAST_THE_END;
 }
 
 // Loader of a tile: lane -> (row lane/4 of a 16-row group, LDS position lane%4); it fetches the
@@ -315,19 +322,17 @@ __device__ __forceinline__ Loader make_loader(const MokGemmResidue& g, const Mok
 #pragma unroll
   for (int i = 0; i < W_GROUPS; ++i) {
     const int wl = (wave * W_GROUPS + i) * 16 + lrow;  // tile-local weight row
-    int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
-    col = col < wv.rows ? col : wv.rows - 1;
-    ld.wsrc[i] = (uint32_t)col * (uint32_t)K_SLOT + chunk;  // weights are K-tiled: [K/64][rows][64]
+    const int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
+    ld.wsrc[i] = col < wv.rows ? (uint32_t)col * (uint32_t)K_SLOT + chunk : PAST_THE_END;  // weights are K-tiled: [K/64][rows][64]
   }
   ld.w = make_rsrc(wv.q + (int64_t)expert * wv.expert_pitch_q, (uint32_t)wv.rows * (uint32_t)wv.k);
   ld.w_slot_pitch = (uint32_t)wv.rows * (uint32_t)K_SLOT;
   // weight scales, slot-major [pair][row][4]: thread tid fetches tile row tid's dword
   static_assert(THREADS == TILE_W, "one thread per weight row");
-  int col = t.col_begin + (gate_up ? (tid & (TILE_W / 2 - 1)) : tid);
-  col = col < wv.rows ? col : wv.rows - 1;
+  const int col = t.col_begin + (gate_up ? (tid & (TILE_W / 2 - 1)) : tid);
   ld.wsc = make_rsrc(wv.sc + (int64_t)expert * wv.expert_pitch_sc,
                      (uint32_t)((wv.k + K_PAIR - 1) / K_PAIR) * (uint32_t)wv.rows * 4u);
-  ld.wscsrc = (uint32_t)col * 4u;
+  ld.wscsrc = col < wv.rows ? (uint32_t)col * 4u : PAST_THE_END;
   ld.wsc_pair_pitch = (uint32_t)wv.rows * 4u;
   return ld;
 }
