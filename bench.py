@@ -11,14 +11,24 @@ metric = MXFP8 grouped-GEMM TFLOP/s on the algorithmic (unpadded) flop count
   cpu_baseline  -- the CPU oracle (torch fp32 dequant-then-matmul) timed on the host cores on
                    the first 1024 tokens of the same inputs;
   linked_over_one_unit -- paired ABBA/BAAB timing of the linked image against the one-unit
-                   control (evaluator/harness/parity/example.py:104-166 in the reference)."""
+                   control (evaluator/harness/parity/example.py:104-166 in the reference);
+  power         -- board power and shader clock the driver reports (hwmon power1_input,
+                   pp_dpm_sclk) sampled while the timed steps run: this kernel runs at the
+                   board's power cap, and the clock it is given there bounds what it can reach.
+
+Before the warm-up steps the forward is looped, untimed, for --ramp-seconds: a GPU that has been
+idle needs about a second of load to reach its sustained clock and power state, and steps timed
+before that are neither the burst nor the sustained rate."""
 from __future__ import annotations
 
 import argparse
+import glob
 import json
 import os
+import re
 import statistics
 import sys
+import threading
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -69,6 +79,58 @@ def make_inputs(dev, seed=0):
     return dev_args, row_major
 
 
+class PowerSampler:
+    """Reads board power (hwmon power1_input, microwatts) and the current shader clock level
+    (pp_dpm_sclk, the line marked with *) every 50 ms on a thread; best effort: a box that
+    does not expose them yields nulls."""
+
+    def __init__(self):
+        hw = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*"))
+        self.power = next((os.path.join(h, "power1_input") for h in hw if os.path.exists(os.path.join(h, "power1_input"))), None)
+        self.cap = next((os.path.join(h, "power1_cap") for h in hw if os.path.exists(os.path.join(h, "power1_cap"))), None)
+        sclk = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+        self.sclk = sclk[0] if sclk else None
+        self.watts, self.mhz = [], []
+        self._stop = threading.Event()
+        self._thread = None
+
+    @staticmethod
+    def _read(path):
+        try:
+            with open(path) as f:
+                return f.read()
+        except OSError:
+            return None
+
+    def _run(self):
+        while not self._stop.is_set():
+            w = self._read(self.power) if self.power else None
+            if w and w.strip().isdigit():
+                self.watts.append(int(w) / 1e6)
+            c = self._read(self.sclk) if self.sclk else None
+            m = re.search(r"(\d+)\s*Mhz\s*\*", c or "", re.IGNORECASE)
+            if m:
+                self.mhz.append(int(m.group(1)))
+            self._stop.wait(0.05)
+
+    def __enter__(self):
+        self._thread = threading.Thread(target=self._run, daemon=True)
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        self._thread.join()
+
+    def report(self):
+        cap = self._read(self.cap) if self.cap else None
+        return {"cap_w": round(int(cap) / 1e6, 1) if cap and cap.strip().isdigit() else None,
+                "draw_w": round(statistics.median(self.watts), 1) if self.watts else None,
+                "sclk_mhz": round(statistics.median(self.mhz)) if self.mhz else None,
+                "samples": len(self.watts),
+                "source": "hwmon power1_input / power1_cap, pp_dpm_sclk, sampled every 50 ms during the timed steps"}
+
+
 def cpu_baseline(inp, row_major, sample_tokens=1024, reps=3):
     """The oracle on the host cores, first `sample_tokens` tokens of the same inputs."""
     import numpy as np
@@ -103,8 +165,10 @@ def cpu_baseline(inp, row_major, sample_tokens=1024, reps=3):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--ramp-seconds", type=float, default=1.5,
+                    help="loop the forward, untimed, for this long before the warm-up steps (clock and power ramp)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-pair", action="store_true", help="skip the linked vs one-unit paired timing")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -143,14 +207,20 @@ def main() -> int:
     stream = torch.cuda.current_stream().cuda_stream
     be = HipBackend(0, stream)
 
+    ramp_end = time.perf_counter() + args.ramp_seconds
+    while time.perf_counter() < ramp_end:
+        for _ in range(50):
+            linked.forward(prob)
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         linked.forward(prob)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        linked.forward(prob)
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    with PowerSampler() as power:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            linked.forward(prob)
+        torch.cuda.synchronize()
+        ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
     def event_ms(sess, which, n):
         e0, e1 = be.event_create(), be.event_create()
@@ -164,9 +234,23 @@ def main() -> int:
         be.event_destroy(e1)
         return ms
 
-    n = max(args.steps, 10)
-    ms_gate_up = event_ms(linked, 1, n)
-    ms_down = event_ms(linked, 2, n)
+    # per-pass launch durations: the forward is launched as its two passes in turn, as above, and
+    # each pass is bracketed by its own pair of events (a loop over one pass alone would keep that
+    # pass's weights in the last-level cache and change the clock the other pass leaves it)
+    n = min(max(args.steps, 10), 200)
+    ev = [[be.event_create() for _ in range(3)] for _ in range(n)]
+    for a, b, c in ev:
+        be.event_record(a)
+        linked.forward(prob, which=1)
+        be.event_record(b)
+        linked.forward(prob, which=2)
+        be.event_record(c)
+    be.event_synchronize(ev[-1][2])
+    ms_gate_up = statistics.mean(be.event_elapsed_time(a, b) for a, b, c in ev)
+    ms_down = statistics.mean(be.event_elapsed_time(b, c) for a, b, c in ev)
+    for trio in ev:
+        for e in trio:
+            be.event_destroy(e)
 
     pair = None
     if not args.no_pair:
@@ -189,7 +273,8 @@ def main() -> int:
         "metric": "MXFP8 MoE grouped-GEMM TFLOP/s (% MFMA peak); linked/one-unit speed ratio",
         "value": round(FLOPS_TOTAL / (ms_per_step * 1e-3) / 1e12, 2),
         "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ramp_seconds": args.ramp_seconds,
+        "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3 (MXFP8, fp32 accumulate)",
         "data": "synthetic",
         "config": {"workload": "configs[2]: MXFP8 MoE expert FFN forward", "tokens": T, "d_model": H, "d_ff": I,
@@ -202,7 +287,14 @@ def main() -> int:
                      "traffic": TRAFFIC_GATE_UP_BYTES, "launch_ms": round(ms_gate_up, 4),
                      "down_pass": {"achieved": round(FLOPS_DOWN / (ms_down * 1e-3) / 1e12, 2), "launch_ms": round(ms_down, 4)}},
         "linked_over_one_unit": pair,
+        "power": power.report(),
     }
+    sclk = out["power"]["sclk_mhz"]
+    if sclk:
+        # the published peak is 256 CUs x 4 SIMDs x 2048 FP8 flop per clock at 2.4 GHz
+        at_clock = PEAK_FP8_TFLOPS * sclk / 2400.0
+        out["roofline"]["peak_at_reported_sclk"] = round(at_clock, 1)
+        out["roofline"]["frac_at_reported_sclk"] = round(FLOPS_GATE_UP / (ms_gate_up * 1e-3) / 1e12 / at_clock, 4)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(inp, row_major)
     print(json.dumps(out))
