@@ -74,6 +74,8 @@ __device__ __forceinline__ void forward(const MokActResidue& p, const MokActTask
   const int wave = tid >> 6;
   const int half = lane >> 5;
   unsigned char* stage = pipelink_smem + pipelink_mok_act_arena();
+  // (a wave whose rows or columns all lie past the end computes on an accumulator the GEMM owner
+  // cleared and did not fill; a branch around the arithmetic for it costs every wave spills)
   // ---- activation + requant into an LDS tile [256 rows][128 codes] + [256 rows][4 scales] ----
 #pragma unroll
   for (int a = 0; a < 2; ++a) {  // gate fragments a, up fragments a + 2: same rows, same columns

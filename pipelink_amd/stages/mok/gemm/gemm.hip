@@ -115,6 +115,18 @@ struct Rings {
 
 __device__ __forceinline__ int swizzle(int row) { return (row >> 2) & 3; }
 
+// A wave whose whole 128 x 128 share of the tile lies past the end of the expert's rows, or past
+// the last output column, has nothing to multiply: it keeps loading its share of the tile's
+// operands for the other waves and meets every barrier, and leaves the matrix pipe and its
+// operand reads alone (the accumulator it hands on is never looked at: its outputs are not
+// stored).  `cols` is the number of output columns (weight rows of one matrix).
+__device__ __forceinline__ bool wave_idle(const MokGemmTask& t, int cols) {
+  const int wave = __builtin_amdgcn_readfirstlane(fresh_tid() >> 6);
+  const bool no_rows = t.row_begin + xrow0(wave, 0) >= t.row_end;
+  const bool no_cols = t.col_begin + wave_w(wave) * 64 >= cols;  // the wave's lowest column, both ops
+  return no_rows || no_cols;
+}
+
 // Issue the weight rows of slot j into weight buffer `buf`, preceded by the scale loads that
 // go with slot j.  Scale loads go first so that they are older than tile loads of the same
 // step: the outstanding-load counts the waits use only count tile loads, which errs on the
@@ -427,6 +439,8 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
     wscoff[a] = wl * 4;
   }
 
+  // cleared for an idle wave as well: an accumulator it left unwritten would be the previous
+  // tile's, kept alive across the loop
 #pragma unroll
   for (int a = 0; a < WFRAGS; ++a)
 #pragma unroll
@@ -444,6 +458,33 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   for (int u = 2 - DEPTH; u < 0; ++u) issue_step(ld, r, u, n, (u + DEPTH) & ~1, ((u + DEPTH) & ~1) + 1, u + DEPTH);
   wait_loads_and_reads_dyn(loads_younger_than_slot<DEPTH>(0, -1, n));
   wg_barrier();
+  auto xnext = [](int b, int by) {  // (b + by) mod XDEPTH for 0 <= b < XDEPTH, 0 <= by <= XDEPTH
+    const int c = b + by;
+    return c >= XDEPTH ? c - XDEPTH : c;
+  };
+  if (wave_idle(t, (gate_up ? g.w_gate : g.w_down).rows)) {
+    // Loader only.  Same loop bounds as the multiplying waves below, one wait + barrier + issue
+    // per step, so every wave of the workgroup passes the same number of barriers.
+    int xb = 0, wb = 0;
+    auto step = [&](int t_) {
+      wait_loads_and_reads_dyn(loads_younger_than_slot<DEPTH>(t_ + 1, t_ - 1, n));
+      wg_barrier();
+      const bool odd_step = t_ & 1;
+      issue_step(ld, r, t_, n, odd_step ? xnext(xb, XDEPTH - 2) : xnext(xb, XDEPTH - 1), odd_step ? xnext(xb, XDEPTH - 1) : xb, wb);
+      xb = xnext(xb, 1);
+      wb = wb + 1 == DEPTH ? 0 : wb + 1;
+    };
+    int j = 0;
+    for (; j + 8 + DEPTH <= n; j += 8)
+      for (int s8 = 0; s8 < 8; ++s8) step(j + s8);
+    for (; j + 1 < n; j += 2) {
+      step(j);
+      step(j + 1);
+    }
+    wg_barrier();
+    return;
+  }
+
   Operands even, odd;
   int sx[XFRAGS], sw[WFRAGS], sxn[XFRAGS], swn[WFRAGS];
   read_operands(even, r.x(0), r.w(0), xoff, woff);
@@ -461,10 +502,6 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   static_assert(8 % DEPTH == 0, "a group of eight slots must start at weight buffer 0");
   int j = 0;
   int xb = 0;  // routed-row buffer of slot j
-  auto xnext = [](int b, int by) {  // (b + by) mod XDEPTH for 0 <= b < XDEPTH, 0 <= by <= XDEPTH
-    const int c = b + by;
-    return c >= XDEPTH ? c - XDEPTH : c;
-  };
   for (; j + 8 + DEPTH <= n; j += 8) {
     auto step = [&](auto S_) {
       constexpr int S = decltype(S_)::value;
@@ -600,7 +637,9 @@ __device__ __forceinline__ void store_down(const MokGemmResidue& g, const MokGem
   const int tid = fresh_tid();
   const int lane = tid & 63;
   const int wave = tid >> 6;
+  const bool idle = wave_idle(t, g.w_down.rows);  // this wave's accumulator holds nothing
   if constexpr (ARENA_BYTES < TILE_X / 2 * Y_PITCH) {
+    if (idle) return;
 #pragma unroll
     for (int b = 0; b < XFRAGS; ++b) {
       const int row = t.row_begin + xrow0(wave, b) + (lane & 31);
@@ -626,7 +665,7 @@ __device__ __forceinline__ void store_down(const MokGemmResidue& g, const MokGem
     const bool col_ok = t.col_begin + chunk * 8 < g.w_down.rows;  // column extents are multiples of 32
 #pragma unroll
     for (int pass = 0; pass < PASSES; ++pass) {
-      if (PASSES == 1 || wave_x(wave) == pass) {
+      if (!idle && (PASSES == 1 || wave_x(wave) == pass)) {
 #pragma unroll
         for (int b = 0; b < XFRAGS; ++b) {
           unsigned char* rowp = stage + (xrow0(wave, b) - pass * ROWS + (lane & 31)) * Y_PITCH;
