@@ -131,6 +131,49 @@ class PowerSampler:
                 "source": "hwmon power1_input / power1_cap, pp_dpm_sclk, sampled every 50 ms during the timed steps"}
 
 
+def mfma_ceiling(be, torch, seconds=1.0):
+    """What back-to-back v_mfma_scale_f32_32x32x64_f8f6f4 alone sustain on this board (one wave per
+    SIMD, operands in registers, no LDS or memory traffic): with random e4m3 operands the board
+    sits at its power limit and clocks down; with zero operands it runs at the full clock."""
+    from pipelink_amd.host.backend import check, load_library
+
+    lib = load_library()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.zeros(16, dtype=torch.float32, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    iters, per_batch = 2000, 20
+    flop_per_launch = cus * 4 * iters * 16 * 131072.0
+    out = {}
+    for name, zero in (("random_operands", 0), ("zero_operands", 1)):
+        def batch():
+            for _ in range(per_batch):
+                check(lib, lib.plk_probe_mfma_fp8(cus, iters, zero, sink.data_ptr(), stream))
+        end = time.perf_counter() + seconds  # clock / power ramp
+        while time.perf_counter() < end:
+            batch()
+            torch.cuda.synchronize()
+        e0, e1 = be.event_create(), be.event_create()
+        launches = 0
+        with PowerSampler() as power:
+            be.event_record(e0)
+            end = time.perf_counter() + seconds
+            while time.perf_counter() < end:
+                batch()
+                launches += per_batch
+                torch.cuda.synchronize()
+            be.event_record(e1)
+            be.event_synchronize(e1)
+        ms = be.event_elapsed_time(e0, e1)
+        be.event_destroy(e0)
+        be.event_destroy(e1)
+        rep = power.report()
+        out[name] = {"tflops": round(flop_per_launch * launches / (ms * 1e-3) / 1e12, 1), "draw_w": rep["draw_w"],
+                     "sclk_mhz": rep["sclk_mhz"], "launches": launches}
+    out["definition"] = (f"plk_probe_mfma_fp8: {cus} workgroups x 4 waves, {iters} x 16 MFMA 32x32x64 f8f6f4 per wave and "
+                         f"launch, operands in registers; {seconds} s ramp then {seconds} s timed with HIP events")
+    return out
+
+
 def cpu_baseline(inp, row_major, sample_tokens=1024, reps=3):
     """The oracle on the host cores, first `sample_tokens` tokens of the same inputs."""
     import numpy as np
@@ -171,6 +214,8 @@ def main() -> int:
                     help="loop the forward, untimed, for this long before the warm-up steps (clock and power ramp)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-pair", action="store_true", help="skip the linked vs one-unit paired timing")
+    ap.add_argument("--no-mfma-ceiling", action="store_true",
+                    help="skip the pure-MFMA run that measures what the matrix pipe sustains at the board's power limit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 1 GiB device copy, 10 times: the known-size kernel the FETCH_SIZE / "
                          "WRITE_SIZE counters are scaled by")
@@ -269,6 +314,10 @@ def main() -> int:
         pair = {"speed_ratio": round(statistics.median(ratios), 5), "blocks": [round(r, 5) for r in ratios],
                 "batch": batch, "definition": "one-unit time / linked time, median of 8 ABBA/BAAB blocks"}
 
+    ceiling = None
+    if not args.no_mfma_ceiling:
+        ceiling = mfma_ceiling(be, torch)
+
     out = {
         "metric": "MXFP8 MoE grouped-GEMM TFLOP/s (% MFMA peak); linked/one-unit speed ratio",
         "value": round(FLOPS_TOTAL / (ms_per_step * 1e-3) / 1e12, 2),
@@ -295,6 +344,10 @@ def main() -> int:
         at_clock = PEAK_FP8_TFLOPS * sclk / 2400.0
         out["roofline"]["peak_at_reported_sclk"] = round(at_clock, 1)
         out["roofline"]["frac_at_reported_sclk"] = round(FLOPS_GATE_UP / (ms_gate_up * 1e-3) / 1e12 / at_clock, 4)
+    if ceiling:
+        out["mfma_ceiling"] = ceiling
+        rnd = ceiling["random_operands"]["tflops"]
+        out["roofline"]["frac_of_measured_mfma_ceiling"] = round(FLOPS_GATE_UP / (ms_gate_up * 1e-3) / 1e12 / rnd, 4)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(inp, row_major)
     print(json.dumps(out))
