@@ -1,0 +1,42 @@
+"""Host side of the three-package GEMM example (C = GELU(A . B + bias)) on the host-less route:
+packs the three stages' params blobs from buffer addresses and opens a ``HostlessSession``.
+
+The reference launches its examples the same way (``pipec2.launcher.open_hostless``,
+launcher.py:201-259; examples/ring-pipeline/run.py): buffers by name, a callable that turns their
+device addresses into per-stage params, the grid."""
+from __future__ import annotations
+
+import struct
+from pathlib import Path
+
+import numpy as np
+
+from ..pipec.launcher import HostlessSession, open_hostless
+
+TILE = 128
+TILE_K = 64
+
+
+def params_blobs(addr: dict[str, int], m: int, n: int, k: int) -> dict[str, bytes]:
+    """GsLoaderParams (40 B), GsMmaParams (16 B), GsEpilogueParams (24 B) of include/gs_abi.h."""
+    return {
+        "gs.loader": struct.pack("<QQQiiii", addr["a"], addr["bt"], addr["status"], m, n, k, 0),
+        "gs.mma": struct.pack("<Qii", addr["status"], n, k),
+        "gs.epilogue": struct.pack("<QQii", addr["bias"], addr["c"], m, n),
+    }
+
+
+def open_session(link_json: str | Path, a_bits: np.ndarray, bt_bits: np.ndarray, bias: np.ndarray, *, backend=None,
+                 image: str | Path | None = None) -> HostlessSession:
+    """a_bits [m,k] and bt_bits [n,k]: bf16 bit patterns (uint16); bias [n] float32.  Buffers: a, bt, bias,
+    c ([m,n] uint16, zeroed), status ([1] uint32: non-zero if a ring wait gave up)."""
+    m, k = a_bits.shape
+    n, k2 = bt_bits.shape
+    if k != k2 or bias.shape != (n,):
+        raise ValueError("operand shapes do not agree")
+    if m % TILE or n % TILE or k % TILE_K or a_bits.dtype != np.uint16 or bt_bits.dtype != np.uint16:
+        raise ValueError("m and n must be multiples of 128, k of 64, operands uint16 bf16 bit patterns")
+    buffers = {"a": a_bits, "bt": bt_bits, "bias": bias.astype(np.float32), "c": ((m, n), np.uint16),
+               "status": ((1,), np.uint32)}
+    return open_hostless(link_json, buffers=buffers, params=lambda addr: params_blobs(addr, m, n, k),
+                         grid=((m // TILE) * (n // TILE),), backend=backend, image=image)

@@ -119,6 +119,9 @@ inline int emit_main() {
 // extent = base + per * value(depth_handle): an LDS ring whose depth is bound at link time
 #define PL_CLAIM_RING(handle, domain, base, depth_handle, per, align, lifetime) \
   PL_REG("claims", "{\"handle\":" + ::pl::quote(handle) + ",\"domain\":" + ::pl::quote(domain) + ",\"extent\":{\"const\":" + ::pl::num(base) + ",\"per\":{" + ::pl::quote(depth_handle) + ":" + ::pl::num(per) + "}},\"align\":" + ::pl::num(align) + ",\"lifetime\":" + ::pl::quote(lifetime) + "}")
+// the waves of role `role`: the handle's value is the index of the role's first wave in the workgroup
+#define PL_CLAIM_WARPS(handle, role, warps) \
+  PL_REG("claims", "{\"handle\":" + ::pl::quote(handle) + ",\"domain\":\"warp\",\"extent\":{\"const\":" + ::pl::num(warps) + ",\"per\":{}},\"align\":1,\"roles\":[" + ::pl::quote(#role) + "],\"lifetime\":\"kernel\"}")
 #define PL_VARIANT(index, ...) \
   PL_REG("variants", "{\"index\":" + ::pl::num(index) + ",\"key\":" + ::pl::keyset(__VA_ARGS__) + "}")
 #define PL_TOPOLOGY(persistent, scheduler) \
@@ -126,6 +129,22 @@ inline int emit_main() {
 // a global-memory counter channel: release add on the producing side, acquire load on the other
 #define PL_COUNTER(name, direction, slot_handle, exports) \
   PL_REG("counters", "{\"name\":" + ::pl::quote(#name) + ",\"direction\":" + ::pl::quote(direction) + ",\"slot\":" + ::pl::quote(slot_handle) + ",\"exports\":" + ::pl::strlist(exports) + "}")
+// One end of an LDS ring with full / empty counters (protocol kind "mbarrier" in the manifest):
+// `direction` "produce" or "consume"; the tile is one ring stage, rows x cols elements of `dtype`
+// (`elem_bits` wide), `stride` bytes apart; `depth` is the depth handle; the full counters live in
+// the slots of handle `full` and take `full_count` arrivals per fill from role `full_by`, the
+// empty counters in `empty` with `empty_count` arrivals per drain from `empty_by` (counts are
+// integers or expressions such as "warps(mma)"); `init_owner` is the role on whose behalf the
+// dispatch kernel zeroes the counters.  Both ends must state the same thing.
+#define PL_RING(name, direction, owner_role, dtype, elem_bits, rows, cols, depth, stride, full, full_count, full_by, empty, \
+                empty_count, empty_by, init_owner)                                                                       \
+  PL_REG("rings", "{\"name\":" + ::pl::quote(#name) + ",\"direction\":" + ::pl::quote(direction) + ",\"owner_role\":" +   \
+                      ::pl::quote(#owner_role) + ",\"dtype\":" + ::pl::quote(dtype) + ",\"elem_bits\":" + ::pl::num(elem_bits) + \
+                      ",\"rows\":" + ::pl::num(rows) + ",\"cols\":" + ::pl::num(cols) + ",\"depth\":" + ::pl::quote(depth) +   \
+                      ",\"stride\":" + ::pl::num(stride) + ",\"full\":" + ::pl::quote(full) + ",\"full_count\":" +           \
+                      ::pl::quote(full_count) + ",\"full_by\":" + ::pl::quote(#full_by) + ",\"empty\":" + ::pl::quote(empty) +  \
+                      ",\"empty_count\":" + ::pl::quote(empty_count) + ",\"empty_by\":" + ::pl::quote(#empty_by) +            \
+                      ",\"init_owner\":" + ::pl::quote(#init_owner) + "}")
 // a published geometry fact of this owner (reaches other owners only through the link)
 #define PL_FACT(name, value) PL_REG("facts", "{\"name\":" + ::pl::quote(name) + ",\"value\":" + ::pl::num(value) + "}")
 // a header whose declarations cross a call seam (task records, fragment types): its text
@@ -148,9 +167,12 @@ inline int emit_main() {
 #define PL_SERVE(channel, export_name)
 #define PL_CLAIM(handle, domain, extent, align, lifetime)
 #define PL_CLAIM_RING(handle, domain, base, depth_handle, per, align, lifetime)
+#define PL_CLAIM_WARPS(handle, role, warps)
 #define PL_VARIANT(index, ...)
 #define PL_TOPOLOGY(persistent, scheduler)
 #define PL_COUNTER(name, direction, slot_handle, exports)
+#define PL_RING(name, direction, owner_role, dtype, elem_bits, rows, cols, depth, stride, full, full_count, full_by, empty, \
+                empty_count, empty_by, init_owner)
 #define PL_FACT(name, value)
 #define PL_USES(handle)
 #define PL_PRELUDE(path)

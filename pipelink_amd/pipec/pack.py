@@ -134,6 +134,24 @@ def assemble(registry: dict[str, Any], profile_name: str, source: Path) -> dict[
             "protocol": {"kind": "counter", "slot": c["slot"], "release": "atomic_add.release.agent",
                          "acquire": "load.acquire.agent"},
             "binds": {}})
+    def count(text: str):
+        return int(text) if text.isdigit() else text
+
+    for r in registry.get("rings", []):
+        endpoints.append({
+            "name": r["name"], "direction": r["direction"], "owner_role": r["owner_role"],
+            "space": "smem", "scope": "cta", "proxy": "async", "tile": {"dtype": r["dtype"], "shape": [r["rows"], r["cols"]]},
+            "layout": {"encoding": "pl-layout-v2", "elem_bits": r["elem_bits"], "shape": [[r["rows"]], [r["cols"]]],
+                       "stride": [[r["cols"]], [1]]},
+            "ring": {"depth": {"handle": r["depth"]}, "stage_stride_bytes": r["stride"]},
+            "protocol": {"kind": "mbarrier",
+                         "full": {"slots": r["full"], "arrive": {"count": count(r["full_count"]), "by": r["full_by"]},
+                                  "tx_bytes": "tile"},
+                         "empty": {"slots": r["empty"], "arrive": {"count": count(r["empty_count"]), "by": r["empty_by"]},
+                                   "tx_bytes": 0},
+                         "init": {"owner": r["init_owner"], "materializer": "dispatch", "phase": 0},
+                         "release": "once-per-acquire"},
+            "binds": {"full": r["full"], "empty": r["empty"]}})
     topo = (registry.get("topology") or [{"persistent": False, "scheduler": "static"}])[0]
     variants = sorted(registry.get("variants") or [{"index": 0, "key": {}}], key=lambda v: v["index"])
     probe = plink.sha256_hex(plink.canonical_bytes({"type": params["type"], "bytes": params["bytes"],
