@@ -227,3 +227,39 @@ def test_full_size_properties(cell):
                                   host.w_up_q.numpy(), host.w_up_sc.numpy(), host.w_down_q.numpy(), host.w_down_sc.numpy(),
                                   one, host.row_token.numpy()[lo:lo + n])
     assert moe_ffn.rel_frobenius(yy[lo:lo + n], ref["y"]) <= TOL
+
+
+def test_benchmark_configuration_properties(cell):
+    """The benchmark's own shape (T=8192, d_model = d_ff = 2880, 32 experts, top-4), where the oracle
+    on every row is too slow for a GPU test: (1) no output is left poisoned; (2) shuffling the routed rows
+    inside every expert shuffles the output rows the same way, byte for byte -- a row's result does not
+    depend on which tile, wave or lane it lands in; (3) the linked image and the one-unit control write the
+    same bytes; (4) one expert's rows against the oracle run on those rows only."""
+    from pipelink_amd.host import mok_inputs
+
+    T, H, I, E, k = 8192, 2880, 2880, 32, 4
+    inp = mok_inputs.generate(T, H, I, E, k, seed=0, quantize_device=torch.device("cuda:0"))
+    host = mok_inputs.MokInputs(**{n: v.cpu() for n, v in inp.__dict__.items()})
+    del inp
+    hq, hsc, y = _run(cell[0], host, H, I)
+    yb = y.view(torch.int16).numpy()
+    assert not np.isnan(y.float().numpy()).any()                                   # (1)
+    counts = host.tokens_per_expert.numpy()
+    assert counts.sum() == T * k
+    offsets = np.concatenate([[0], np.cumsum(counts)])
+    rng = np.random.default_rng(0)
+    perm = np.concatenate([offsets[e] + rng.permutation(int(counts[e])) for e in range(E)])
+    shuffled = mok_inputs.MokInputs(**{**host.__dict__, "row_token": host.row_token[torch.from_numpy(perm)]})
+    hq2, hsc2, y2 = _run(cell[0], shuffled, H, I)
+    assert np.array_equal(y2.view(torch.int16).numpy(), yb[perm])                  # (2)
+    assert np.array_equal(hq2, hq[perm]) and np.array_equal(hsc2[:, :I // 32], hsc[perm][:, :I // 32])
+    _, _, y3 = _run(cell[1], host, H, I)
+    assert np.array_equal(y3.view(torch.int16).numpy(), yb)                        # (3)
+    e = int(np.argmin(counts))                                                      # (4) the smallest expert
+    lo, n = int(offsets[e]), int(counts[e])
+    one = np.zeros_like(counts)
+    one[e] = n
+    ref = moe_ffn.moe_ffn_forward(host.x_q.numpy(), host.x_sc.numpy(), host.w_gate_q.numpy(), host.w_gate_sc.numpy(),
+                                  host.w_up_q.numpy(), host.w_up_sc.numpy(), host.w_down_q.numpy(), host.w_down_sc.numpy(),
+                                  one, host.row_token.numpy()[lo:lo + n])
+    assert moe_ffn.rel_frobenius(y.float().numpy()[lo:lo + n], ref["y"]) <= TOL
