@@ -6,24 +6,15 @@ launcher.py:201-259; examples/ring-pipeline/run.py): buffers by name, a callable
 device addresses into per-stage params, the grid."""
 from __future__ import annotations
 
-import struct
 from pathlib import Path
 
 import numpy as np
 
 from ..pipec.launcher import HostlessSession, open_hostless
+from ..stages.gemm_split.params import params_blobs
 
 TILE = 128
 TILE_K = 64
-
-
-def params_blobs(addr: dict[str, int], m: int, n: int, k: int) -> dict[str, bytes]:
-    """GsLoaderParams (40 B), GsMmaParams (16 B), GsEpilogueParams (24 B) of include/gs_abi.h."""
-    return {
-        "gs.loader": struct.pack("<QQQiiii", addr["a"], addr["bt"], addr["status"], m, n, k, 0),
-        "gs.mma": struct.pack("<Qii", addr["status"], n, k),
-        "gs.epilogue": struct.pack("<QQii", addr["bias"], addr["c"], m, n),
-    }
 
 
 def open_session(link_json: str | Path, a_bits: np.ndarray, bt_bits: np.ndarray, bias: np.ndarray, *, backend=None,
@@ -40,3 +31,4 @@ def open_session(link_json: str | Path, a_bits: np.ndarray, bt_bits: np.ndarray,
                "status": ((1,), np.uint32)}
     return open_hostless(link_json, buffers=buffers, params=lambda addr: params_blobs(addr, m, n, k),
                          grid=((m // TILE) * (n // TILE),), backend=backend, image=image)
+

@@ -139,3 +139,61 @@ def run_hostless(link_json, *, buffers, params, grid, outputs: list[str], **kw) 
         return {n: s.read(n) for n in outputs}
     finally:
         s.close()
+
+
+def _parse_buffer(spec: str):
+    """``FILE.npy`` or ``SHAPE:DTYPE`` (e.g. ``64x64:float32``, a zeroed buffer)."""
+    if spec.endswith(".npy"):
+        return np.load(spec, allow_pickle=False)
+    shape, _, dtype = spec.partition(":")
+    try:
+        return tuple(int(d) for d in shape.split("x")), np.dtype(dtype)
+    except (ValueError, TypeError):
+        _fail("L-LAUNCH", "launch.buffers", "buffer spec must be FILE.npy or SHAPE:DTYPE", spec=spec)
+
+
+def _load_params_function(spec: str) -> Callable[[dict[str, int]], dict[str, bytes]]:
+    """``PY_FILE:FUNCTION`` -> the function (the file is executed as a module of its own)."""
+    import importlib.util
+
+    path, _, name = spec.rpartition(":")
+    if not path or not name:
+        _fail("L-LAUNCH", "launch.params", "params builder must be PY_FILE:FUNCTION", spec=spec)
+    module_spec = importlib.util.spec_from_file_location("pipec_launch_params", path)
+    if module_spec is None or module_spec.loader is None:
+        _fail("L-LAUNCH", "launch.params", "params builder file cannot be loaded", path=path)
+    module = importlib.util.module_from_spec(module_spec)
+    module_spec.loader.exec_module(module)
+    if not callable(getattr(module, name, None)):
+        _fail("L-LAUNCH", "launch.params", "params builder function not found", function=name)
+    return getattr(module, name)
+
+
+def launch(link_json: str | Path, *, grid: tuple[int, ...] | None, buffers: dict[str, str] | None = None,
+           params: str | None = None, blobs: dict[str, str | Path] | None = None, outputs: dict[str, str | Path] | None = None,
+           providers: dict[str, str] | None = None, device: int = 0, backend=None) -> dict[str, Any]:
+    """One launch on the host-less route, as ``pipec launch`` runs it (pipec/src/pipec2/launcher.py:284-333
+    in the reference): buffers from ``NAME -> FILE.npy | SHAPE:DTYPE``, params either from a Python
+    builder ``PY_FILE:FUNCTION`` (device addresses -> stage bytes) or from ready-made blobs
+    ``STAGE_ID -> file``; named buffers are saved as .npy afterwards.  Returns the report the CLI prints."""
+    if providers:
+        _fail("L-LAUNCH", "launch.providers", "links with host providers are opened through the host broker, not this route")
+    if grid is None:
+        _fail("L-LAUNCH", "launch.grid", "host-less launch requires a grid")
+    if params is not None and blobs:
+        _fail("L-LAUNCH", "launch.params", "params builder and blob paths are mutually exclusive")
+    builder = _load_params_function(params) if params is not None else (
+        lambda addresses: {sid: Path(path).read_bytes() for sid, path in (blobs or {}).items()})
+    parsed = {name: _parse_buffer(spec) for name, spec in (buffers or {}).items()}
+    unknown = sorted(set(outputs or {}) - set(parsed))
+    if unknown:
+        _fail("L-LAUNCH", "launch.outputs", "output names a buffer that was not declared", names=unknown)
+    result = run_hostless(link_json, buffers=parsed, params=builder, grid=tuple(grid), outputs=list(outputs or {}),
+                          backend=backend, device=device)
+    for name, path in (outputs or {}).items():
+        with Path(path).open("wb") as stream:
+            np.save(stream, result[name], allow_pickle=False)
+    link = json.loads(Path(link_json).read_text())
+    g = tuple(grid) + (1,) * (3 - len(grid))
+    return {"geometry": {"grid": list(g), "block": [link["threads"], 1, 1], "dynamic_smem_bytes": link["dyn_smem_bytes"]},
+            "outputs": {name: str(path) for name, path in (outputs or {}).items()}}

@@ -161,7 +161,7 @@ def test_other_mismatches_of_the_pair_are_named_too(example, tmp_path):
 
 @needs_rocm
 def test_params_blobs_have_the_packed_sizes(example):
-    from pipelink_amd.host.gemm_split import params_blobs
+    from pipelink_amd.stages.gemm_split.params import params_blobs
 
     link = json.loads((example[0] / "link" / "link.json").read_text())
     blobs = params_blobs({"a": 1, "bt": 2, "bias": 3, "c": 4, "status": 5}, 512, 512, 512)
@@ -227,4 +227,54 @@ def test_ring_depth_two_gives_the_same_bytes(tmp_path):
     assert np.array_equal(out[0], out[1])
     want = gg.gemm_bias_gelu_torch(a, b, bias).float().numpy()
     got = torch.from_numpy(out[0].view(np.int16)).view(torch.bfloat16).float().numpy()
+    assert (gg.bf16_ulp_distance(got, want, floor=2.0 ** -12) > 1.0).sum() == 0
+
+
+@needs_rocm
+def test_launch_verb_checks_its_arguments_before_touching_a_device(example, tmp_path):
+    from pipelink_amd.pipec import launcher
+    from pipelink_amd.pipec.clauses import LaunchError
+
+    link = example[0] / "link" / "link.json"
+    with pytest.raises(LaunchError) as err:
+        launcher.launch(link, grid=None)
+    assert str(err.value) == "[L-LAUNCH] launch.grid: host-less launch requires a grid"
+    with pytest.raises(LaunchError) as err:
+        launcher.launch(link, grid=(16,), providers={"gs": "libx.so"})
+    assert err.value.failures[0].path == "launch.providers"
+    with pytest.raises(LaunchError) as err:
+        launcher.launch(link, grid=(16,), params="x.py:f", blobs={"gs.mma": "b.bin"})
+    assert "mutually exclusive" in str(err.value)
+    with pytest.raises(LaunchError) as err:
+        launcher.launch(link, grid=(16,), buffers={"c": "512x512:uint16"}, outputs={"d": str(tmp_path / "d.npy")})
+    assert err.value.failures[0].path == "launch.outputs"
+    with pytest.raises(LaunchError) as err:
+        launcher.launch(link, grid=(16,), buffers={"c": "512by512"})
+    assert err.value.failures[0].path == "launch.buffers"
+    builder = launcher._load_params_function(str(ROOT / "pipelink_amd" / "stages" / "gemm_split" / "params.py") + ":params_512")
+    assert set(builder({"a": 1, "bt": 2, "bias": 3, "c": 4, "status": 5})) == {"gs.loader", "gs.mma", "gs.epilogue"}
+
+
+@pytest.mark.gpu
+def test_cli_launch_verb_runs_the_example(tmp_path):
+    import subprocess
+    import sys
+
+    paths = gs_build.images()
+    a, b, bias = gg.inputs()
+    np.save(tmp_path / "a.npy", _bits(a))
+    np.save(tmp_path / "bt.npy", _bits(b.t()))
+    np.save(tmp_path / "bias.npy", bias.numpy())
+    cmd = [sys.executable, "-m", "pipelink_amd.pipec", "launch", str(paths["link_json"]), "--grid", "16",
+           "--buffer", f"a={tmp_path / 'a.npy'}", "--buffer", f"bt={tmp_path / 'bt.npy'}", "--buffer", f"bias={tmp_path / 'bias.npy'}",
+           "--buffer", "c=512x512:uint16", "--buffer", "status=1:uint32",
+           "--params", str(ROOT / "pipelink_amd" / "stages" / "gemm_split" / "params.py") + ":params_512",
+           "--output", f"c={tmp_path / 'c.npy'}", "--output", f"status={tmp_path / 'status.npy'}"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, cwd=ROOT, timeout=120)
+    assert proc.returncode == 0, proc.stderr
+    report = json.loads(proc.stdout)
+    assert report["geometry"] == {"grid": [16, 1, 1], "block": [320, 1, 1], "dynamic_smem_bytes": 131200}
+    assert np.load(tmp_path / "status.npy")[0] == 0
+    got = torch.from_numpy(np.load(tmp_path / "c.npy").view(np.int16)).view(torch.bfloat16).float().numpy()
+    want = gg.gemm_bias_gelu_torch(a, b, bias).float().numpy()
     assert (gg.bf16_ulp_distance(got, want, floor=2.0 ** -12) > 1.0).sum() == 0
