@@ -90,6 +90,27 @@ def test_forward_matches_oracle(cell, T, H, I, E, k, seed, conc):
     assert (hsc[:, :nb] != ref["hidden_sc"][:, :nb]).mean() < 1e-3   # block scales agree except at exact ties
 
 
+def _random_cases(n, seed):
+    """Seeded shapes around the tile edges: row counts that leave whole waves without rows, column
+    counts that leave whole waves without columns, contraction lengths with odd and even slot
+    counts, experts with no tokens."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(n):
+        E = int(rng.integers(1, 10))
+        k = int(rng.integers(1, min(E, 4) + 1))
+        conc = int(rng.integers(1, E + 1)) if rng.random() < 0.3 and E > 1 else 0
+        if conc and conc < k:
+            conc = k
+        cases.append((int(rng.integers(1, 640)), 64 * int(rng.integers(1, 9)), 64 * int(rng.integers(1, 11)), E, k, 100 + i, conc))
+    return cases
+
+
+@pytest.mark.parametrize("T,H,I,E,k,seed,conc", _random_cases(16, 7))
+def test_forward_matches_oracle_on_seeded_random_shapes(cell, T, H, I, E, k, seed, conc):
+    test_forward_matches_oracle(cell, T, H, I, E, k, seed, conc)
+
+
 def test_linked_and_one_unit_images_are_byte_identical(cell):
     from pipelink_amd.host import mok_inputs
 
