@@ -141,6 +141,30 @@ def test_swiglu_limit_is_a_run_time_value(cell):
     assert moe_ffn.rel_frobenius(y.float().numpy(), ref["y"]) <= TOL
 
 
+def test_unclamped_link_variant_matches_the_unclamped_oracle():
+    """Clamp on / off is chosen when the pipeline is linked (variant handle pipelink_mok_clamp): the image
+    linked with 0 must follow the oracle without the clamp, and differ from the clamped result where
+    gate or up exceed the limit."""
+    from pipelink_amd.host import mok_inputs
+    from pipelink_amd.host.mok import MoKSession
+    from pipelink_amd.stages.mok import build as mok_build
+
+    paths = {"link_json": mok_build.HERE / "build_unclamped" / "link" / "link.json",
+             "linked": mok_build.HERE / "build_unclamped" / "link" / "pipeline.hsaco"}
+    assert paths["linked"].exists(), "unclamped image is not built: run __graft_entry__.build()"
+    link = json.loads(paths["link_json"].read_text())
+    assert link["bindings"]["pipelink_mok_clamp"] == [0, "forced"]
+    inp = mok_inputs.generate(200, 256, 192, 3, 2, seed=9)
+    inp.w_gate_sc = (inp.w_gate_sc.to(torch.int16) + 3).to(torch.uint8)   # weights x 8: gate and up well beyond the limit
+    inp.w_up_sc = (inp.w_up_sc.to(torch.int16) + 3).to(torch.uint8)
+    with MoKSession(paths["linked"].read_bytes(), link) as sess:
+        hq, hsc, y = _run(sess, inp, 256, 192, limit=1.0)
+    free = _oracle(inp, limit=None)
+    clamped = _oracle(inp, limit=1.0)
+    assert moe_ffn.rel_frobenius(y.float().numpy(), free["y"]) <= TOL
+    assert moe_ffn.rel_frobenius(clamped["y"], free["y"]) > 10 * TOL      # the two oracles differ by far more than the bar
+
+
 def test_device_quantiser_is_bit_exact():
     from pipelink_amd.host.mok import mxfp8_quantize_device
 
