@@ -4,6 +4,7 @@ import json
 import os
 
 import numpy as np
+import pytest
 import torch
 
 from oracle import moe_ffn, mxfp8
@@ -102,3 +103,23 @@ def test_seed0_routing_histogram_fixture():
         want = json.load(fh)
     assert counts.tolist() == want["tokens_per_expert"]
     assert int(row_token[:8].sum()) == want["row_token_first8_sum"] and counts.sum() == 32768
+
+
+def test_harness_error_reports_follow_their_definitions():
+    from pipelink_amd.host import mok_inputs
+
+    ref = np.array([[1.0, -2.0], [4.0, 0.0]], dtype=np.float32)
+    got = np.array([[1.5, -2.0], [3.0, 0.25]], dtype=np.float32)
+    mean, maximum, relative = mok_inputs.error_stats(ref, got)
+    assert mean == pytest.approx((0.5 + 0 + 1.0 + 0.25) / 4) and maximum == 1.0
+    assert relative == pytest.approx(1.75 / 7.0)
+    assert mok_inputs.error_stats(ref, got, chunk=3) == pytest.approx((mean, maximum, relative))   # chunking changes nothing
+    rep = mok_inputs.tolerance_report(ref, got)
+    assert rep["passed"] is False and rep["abs_max"] == 1.0 and rep["relative_tolerance"] == 1e-2   # 1.0 > 5e-1
+    assert mok_inputs.tolerance_report(ref, ref)["passed"] is True
+    assert mok_inputs.tolerance_report(ref, np.full_like(ref, np.nan))["passed"] is False           # NaN never passes
+    assert mok_inputs.error_stats(np.zeros(3), np.zeros(3)) == (0.0, 0.0, 0.0)
+    a = torch.arange(6, dtype=torch.bfloat16).reshape(2, 3)
+    assert mok_inputs.bitwise_report(a, a.clone()) and not mok_inputs.bitwise_report(a, a + 1)
+    assert not mok_inputs.bitwise_report(a, a.reshape(3, 2).t())                                     # same values, other layout
+    assert mok_inputs.bitwise_report(np.float32([0.0]), np.float32([0.0])) and not mok_inputs.bitwise_report(np.float32([0.0]), np.float32([-0.0]))
