@@ -11,7 +11,6 @@ namespace mok {
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v2i __attribute__((ext_vector_type(2)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 // ---- tile geometry published by the GEMM owner (facts mok.gemm.*) -------------------
@@ -55,17 +54,7 @@ __device__ __forceinline__ int wrow0(int wave, int a) {
 }
 __device__ __forceinline__ int xrow0(int wave, int b) { return wave_x(wave) * 128 + b * 32; }
 
-typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
-
-// 16 bytes per lane, global -> LDS, lane i lands at lds + 16*i
-__device__ __forceinline__ void load16_to_lds(const uint8_t* g, unsigned char* lds) {
-  __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)lds, 16, 0, 0);
-}
-// 4 bytes per lane, lane i lands at lds + 4*i
-__device__ __forceinline__ void load4_to_lds(const uint8_t* g, unsigned char* lds) {
-  __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)lds, 4, 0, 0);
-}
 
 // threadIdx.x as a value the compiler cannot merge with an earlier copy: code that runs after
 // a register-hungry loop derives its lane indices from this, so they are computed where they
@@ -74,12 +63,6 @@ __device__ __forceinline__ int fresh_tid() {
   int t = threadIdx.x;
   asm volatile("" : "+v"(t));
   return t;
-}
-
-__device__ __forceinline__ float bf16_round(float x) {
-  uint32_t u = __float_as_uint(x);
-  u = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
-  return __uint_as_float(u);
 }
 
 }  // namespace mok
