@@ -64,3 +64,25 @@ def bf16_ulp_distance(x: np.ndarray, y: np.ndarray, floor: float = 2.0 ** -126) 
     mag = np.maximum(np.abs(x), np.abs(y)).astype(np.float32)
     expo = np.floor(np.log2(np.maximum(mag, np.float32(floor))))
     return np.abs(x.astype(np.float64) - y.astype(np.float64)) / np.exp2(expo - 7)
+
+
+# ---- one epilogue, many producers: C = (A . B) * scale[col] + bias[col] -----------------------------------
+# (examples/one-epilogue-many-producers/consumer/epilogue.cu:62-69 in the reference computes
+# acc * scale + bias with a per-row scale and a ReLU; the case evaluated here is the per-column scale
+# without an activation.)  Pins: against the library matmul on a small case; linearity in scale and bias.
+
+def scale_bias_inputs(m: int, n: int, k: int, seed: int = 0):
+    """(A [m,k] bf16, B [k,n] bf16, scale [n], bias [n]); A and B from N(0,1) * 0.02; draw order A, B, scale, bias."""
+    g = torch.Generator().manual_seed(seed)
+    a = (torch.randn(m, k, generator=g) * 0.02).to(torch.bfloat16)
+    b = (torch.randn(k, n, generator=g) * 0.02).to(torch.bfloat16)
+    scale = 1.0 + torch.randn(n, generator=g) * 0.1
+    bias = torch.randn(n, generator=g) * 0.1
+    return a, b, scale, bias
+
+
+def gemm_scale_bias_torch(a: torch.Tensor, b: torch.Tensor, scale: torch.Tensor, bias: torch.Tensor,
+                          rows: torch.Tensor | None = None) -> torch.Tensor:
+    """fp32 matmul, then * scale + bias per column, rounded to bf16; `rows` restricts it to a sample of rows."""
+    a = a if rows is None else a[rows]
+    return ((a.float() @ b.float()) * scale.float() + bias.float()).to(torch.bfloat16)

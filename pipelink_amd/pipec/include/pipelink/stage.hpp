@@ -145,6 +145,21 @@ inline int emit_main() {
                       ::pl::quote(full_count) + ",\"full_by\":" + ::pl::quote(#full_by) + ",\"empty\":" + ::pl::quote(empty) +  \
                       ",\"empty_count\":" + ::pl::quote(empty_count) + ",\"empty_by\":" + ::pl::quote(#empty_by) +            \
                       ",\"init_owner\":" + ::pl::quote(#init_owner) + "}")
+// A tile this stage hands to whoever imports tensor `result`: `home` is "agpr", "vgpr" or "lds"; `layout`
+// is "mfma32x32c" (registers: the frame handed over is rows * cols / 64 floats per lane) or "row_major"
+// (lds: `row_pitch` bytes between rows of the wave's tile; 0 for register homes).  rows x cols is one
+// participant's (one wave's) share.
+#define PL_EXPORT_TENSOR(name, result, dtype, rows, cols, home, layout, row_pitch)                                         \
+  PL_REG("tensor_exports", "{\"name\":" + ::pl::quote(#name) + ",\"result\":" + ::pl::quote(result) + ",\"dtype\":" +      \
+                               ::pl::quote(dtype) + ",\"shape\":[" + ::pl::num(rows) + "," + ::pl::num(cols) + "],\"home\":" + \
+                               ::pl::quote(home) + ",\"layout\":" + ::pl::quote(layout) + ",\"row_pitch_bytes\":" +        \
+                               ::pl::num(row_pitch) + "}")
+// This stage reads tensor `result` through the link-generated `fn(const void* source, float* dest)` (with
+// `fn_ready()` before it and `fn_done()` after it), which delivers the elements in `layout`.
+#define PL_IMPORT_TENSOR(name, fn, result, dtype, rows, cols, layout)                                                      \
+  PL_REG("tensor_imports", "{\"name\":" + ::pl::quote(#name) + ",\"fn\":" + ::pl::quote(#fn) + ",\"result\":" +           \
+                               ::pl::quote(result) + ",\"dtype\":" + ::pl::quote(dtype) + ",\"shape\":[" + ::pl::num(rows) + \
+                               "," + ::pl::num(cols) + "],\"layout\":" + ::pl::quote(layout) + "}")
 // a published geometry fact of this owner (reaches other owners only through the link)
 #define PL_FACT(name, value) PL_REG("facts", "{\"name\":" + ::pl::quote(name) + ",\"value\":" + ::pl::num(value) + "}")
 // a header whose declarations cross a call seam (task records, fragment types): its text
@@ -173,6 +188,8 @@ inline int emit_main() {
 #define PL_COUNTER(name, direction, slot_handle, exports)
 #define PL_RING(name, direction, owner_role, dtype, elem_bits, rows, cols, depth, stride, full, full_count, full_by, empty, \
                 empty_count, empty_by, init_owner)
+#define PL_EXPORT_TENSOR(name, result, dtype, rows, cols, home, layout, row_pitch)
+#define PL_IMPORT_TENSOR(name, fn, result, dtype, rows, cols, layout)
 #define PL_FACT(name, value)
 #define PL_USES(handle)
 #define PL_PRELUDE(path)

@@ -30,6 +30,7 @@ from .clauses import ClauseFailure, LinkError, PipeLinkError
 from .glue import KERNEL_SYMBOL, collect_preludes, generate_dispatch, generate_stub, params_layout
 from .manifest import Pipeline, Stage, load_pipeline, load_stage_manifest, validate_assembly
 from .pack import DEVICE_FLAGS, HIPCC, INCLUDE_DIR, LLVM_BIN
+from .tensors import generate_adapters, plan_connections
 from .solver import solve
 
 
@@ -136,8 +137,11 @@ def link(pipeline_path: str | Path, out_dir: str | Path, *, include_dirs: list[s
     out_dir.mkdir(parents=True, exist_ok=True)
     pipeline, stages, payloads, hashes = load_assembly(pipeline_path)
     channels, expansions, solution, layout = plan(pipeline, stages)
+    tensor_plans = plan_connections(pipeline, stages)
     arch = pipeline.profile.name
     stub = generate_stub(pipeline, stages, channels, expansions, solution, layout)
+    if tensor_plans:
+        stub += "\n#include <hip/hip_runtime.h>\n" + generate_adapters(tensor_plans)
     dispatch = generate_dispatch(pipeline, stages, expansions, solution, layout)
     (out_dir / "prelude").mkdir(exist_ok=True)
     for name, text in collect_preludes(stages).items():
@@ -182,6 +186,7 @@ def link(pipeline_path: str | Path, out_dir: str | Path, *, include_dirs: list[s
         "intervals": {d: [i.to_json_obj() for i in iv] for d, iv in sorted(solution.intervals.items())},
         "roles": {r: {"stage": s, "first_warp": lo, "warps": n} for r, (s, lo, n) in sorted(solution.role_warps.items())},
         "protocol_expansions": [e.to_json_obj() for e in expansions],
+        "tensor_plans": [t.to_json_obj() for t in tensor_plans],
         "facts": {k: v for s in stages for k, v in sorted((s.manifest.get("facts") or {}).items())},
         "observed": observed,
         "input_hashes": hashes,

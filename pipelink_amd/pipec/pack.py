@@ -156,7 +156,12 @@ def assemble(registry: dict[str, Any], profile_name: str, source: Path) -> dict[
     variants = sorted(registry.get("variants") or [{"index": 0, "key": {}}], key=lambda v: v["index"])
     probe = plink.sha256_hex(plink.canonical_bytes({"type": params["type"], "bytes": params["bytes"],
                                                     "align": params["align"]}))
+    tensor = {}
+    if registry.get("tensor_exports") or registry.get("tensor_imports"):
+        tensor = {"tensor": {"schema": "tensor-v1", "exports": registry.get("tensor_exports", []),
+                             "imports": registry.get("tensor_imports", [])}}
     return {
+        **tensor,
         "pipelink_abi": {"schema": "3.0", "target": {
             "profile": profile.name, "lto_arch": profile.lto_arch, "toolkit": TOOLKIT,
             "math": {"flags": DEVICE_FLAGS}}},

@@ -1,0 +1,149 @@
+"""Tensor connections: handing a producer's tile to a consumer that does not know where it lives.
+
+A producer package exports a tensor (``PL_EXPORT_TENSOR``): its logical identity (result name, dtype,
+per-participant shape) and its placement -- the *home* (``agpr``, ``vgpr`` or ``lds``) and the layout in
+that home.  A consumer package imports one (``PL_IMPORT_TENSOR``): the same identity, the layout it wants
+the elements in, and the name of a function it calls to get them.  The pipeline connects an export to an
+import (``tensor_connections``); the linker checks the identities (``T-CONTRACT``), picks a route
+(``T-PLAN`` if none exists) and *generates* the function, together with ``<fn>_ready()`` and
+``<fn>_done()``, into the binding stubs.  The consumer's source never changes with the producer's home.
+
+The reference plans such routes with a model of typed transport primitives and a bounded search
+(pipec/src/pipec2/tensor/plan.py:557 ``ConnectionPlanner``, lowering in tensor/lower.py:679; contract in
+docs/reference/tensor-imports.md:40-142).  On gfx950 the homes an MFMA accumulator can have are three and
+the primitives that read them are fixed, so the planner here is a route table:
+
+    home   layout        route             what the generated function does per element
+    vgpr   mfma32x32c    register_copy     a move the compiler folds away
+    agpr   mfma32x32c    accvgpr_receipt   v_accvgpr_read_b32 from the accumulator register
+    lds    row_major     lds_load          ds_read_b32 at row * pitch + 4 * column of the wave's tile
+
+``mfma32x32c`` is the C/D fragment layout of the 32x32 MFMAs for a tile of rows x cols split into 32 x 32
+blocks [i][j]: element (block i, block j, register r, lane l) is row 32 i + 8 (r / 4) + 4 (l / 32) + r % 4,
+column 32 j + l % 32; in memory order it is word (i * (cols / 32) + j) * 16 + r of the lane's frame.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any
+
+from .clauses import CLAUSES, ClauseFailure, LinkError, register_clause
+from .manifest import Pipeline, Stage
+
+for _cid, _desc in (("T-PLAN", "a transport route exists for every tensor connection"),):
+    if _cid not in CLAUSES:
+        register_clause(_cid, phase="link", description=_desc)
+
+ROUTES = {("vgpr", "mfma32x32c"): "register_copy", ("agpr", "mfma32x32c"): "accvgpr_receipt", ("lds", "row_major"): "lds_load"}
+WANTED_LAYOUTS = ("mfma32x32c",)
+_IDENTITY = ("result", "dtype", "shape")
+
+
+@dataclass(frozen=True)
+class TensorPlan:
+    name: str
+    producer: str
+    consumer: str
+    export: dict[str, Any]
+    imported: dict[str, Any]
+    route: str
+
+    def to_json_obj(self) -> dict[str, Any]:
+        return {"name": self.name, "producer": self.producer, "consumer": self.consumer, "export": self.export["name"],
+                "import": self.imported["name"], "function": self.imported["fn"], "home": self.export["home"],
+                "route": self.route}
+
+
+def _records(stage: Stage, kind: str) -> dict[str, dict[str, Any]]:
+    return {r["name"]: r for r in (stage.manifest.get("tensor") or {}).get(kind, [])}
+
+
+def plan_connections(pipeline: Pipeline, stages: list[Stage]) -> list[TensorPlan]:
+    """One plan per entry of ``pipeline.tensor_connections``; raises LinkError with T-CONTRACT / T-PLAN."""
+    by_id = {s.id: s for s in stages}
+    failures: list[ClauseFailure] = []
+    plans: list[TensorPlan] = []
+    seen_imports: set[tuple[str, str]] = set()
+    for conn in pipeline.body.get("tensor_connections", []) or []:
+        path = f"pipeline.tensor_connections.{conn.get('name', '?')}"
+
+        def bad(clause: str, message: str, **detail: Any) -> None:
+            failures.append(ClauseFailure(clause, path, message, detail))
+
+        prod, cons = by_id.get(conn.get("producer")), by_id.get(conn.get("consumer"))
+        if prod is None or cons is None:
+            bad("T-CONTRACT", "connection names a stage that is not in the pipeline")
+            continue
+        exp = _records(prod, "exports").get(conn.get("export"))
+        imp = _records(cons, "imports").get(conn.get("import"))
+        if exp is None or imp is None:
+            bad("T-CONTRACT", "connection names an export or import its stage does not declare",
+                export=conn.get("export"), imported=conn.get("import"))
+            continue
+        if (cons.id, imp["name"]) in seen_imports:
+            bad("T-CONTRACT", "an import is fed by more than one connection")
+            continue
+        seen_imports.add((cons.id, imp["name"]))
+        differing = [k for k in _IDENTITY if exp.get(k) != imp.get(k)]
+        if differing:
+            bad("T-CONTRACT", "exported and imported tensor identities disagree",
+                fields=differing, exported={k: exp.get(k) for k in differing}, imported={k: imp.get(k) for k in differing})
+            continue
+        rows, cols = exp["shape"]
+        if imp["layout"] not in WANTED_LAYOUTS or rows % 32 or cols % 32:
+            bad("T-PLAN", "no transport route delivers the demanded layout", wanted=imp["layout"], shape=exp["shape"])
+            continue
+        route = ROUTES.get((exp["home"], exp["layout"]))
+        if route is None:
+            bad("T-PLAN", "no transport route reads this home and layout", home=exp["home"], layout=exp["layout"])
+            continue
+        if route == "lds_load" and (exp.get("row_pitch_bytes", 0) < cols * 4 or exp["row_pitch_bytes"] % 4):
+            bad("T-CONTRACT", "row pitch of the exported tile is smaller than a row or not a multiple of 4")
+            continue
+        plans.append(TensorPlan(conn["name"], prod.id, cons.id, exp, imp, route))
+    declared = {(s.id, name) for s in stages for name in _records(s, "imports")}
+    for sid, name in sorted(declared - seen_imports):
+        failures.append(ClauseFailure("T-CONTRACT", f"stages.{sid}.tensor.imports.{name}",
+                                      "import is not fed by any tensor connection"))
+    if failures:
+        raise LinkError(failures)
+    return plans
+
+
+def generate_adapters(plans: list[TensorPlan]) -> str:
+    """HIP source of the generated import functions (appended to the binding stubs)."""
+    out: list[str] = []
+    for p in plans:
+        fn = p.imported["fn"]
+        rows, cols = p.export["shape"]
+        bi, bj = rows // 32, cols // 32
+        out += [f"// tensor connection {p.name}: {p.producer}.{p.export['name']} ({p.export['home']}, {p.export['layout']}) -> "
+                f"{p.consumer}.{p.imported['name']} ({p.imported['layout']}); route {p.route}",
+                f'extern "C" __device__ __attribute__((always_inline)) void {fn}_ready() {{ asm volatile("" ::: "memory"); }}']
+        if p.route == "lds_load":
+            out.append(f'extern "C" __device__ __attribute__((always_inline)) void {fn}_done() {{ '
+                       '__builtin_amdgcn_s_waitcnt(0xC07F); asm volatile("" ::: "memory"); }  // the tile has been read')
+        else:
+            out.append(f'extern "C" __device__ __attribute__((always_inline)) void {fn}_done() {{ asm volatile("" ::: "memory"); }}')
+        out.append(f'extern "C" __device__ __attribute__((always_inline)) void {fn}(const void* source, float* dest) {{')
+        if p.route == "register_copy":
+            out += ["  const float* frame = static_cast<const float*>(source);", "#pragma unroll",
+                    f"  for (int k = 0; k < {bi * bj * 16}; ++k) dest[k] = frame[k];"]
+        elif p.route == "accvgpr_receipt":
+            out += ["  const float* frame = static_cast<const float*>(source);", "#pragma unroll",
+                    f"  for (int k = 0; k < {bi * bj * 16}; ++k) {{",
+                    "    float v;",
+                    '    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(frame[k]));',
+                    "    dest[k] = v;", "  }"]
+        else:
+            pitch = p.export["row_pitch_bytes"]
+            out += ["  const unsigned char* tile = static_cast<const unsigned char*>(source);",
+                    "  const int lane = threadIdx.x & 63;", "#pragma unroll",
+                    f"  for (int i = 0; i < {bi}; ++i)", "#pragma unroll",
+                    f"    for (int j = 0; j < {bj}; ++j)", "#pragma unroll",
+                    "      for (int r = 0; r < 16; ++r) {",
+                    "        const int row = 32 * i + 8 * (r / 4) + 4 * (lane >> 5) + r % 4, col = 32 * j + (lane & 31);",
+                    f"        dest[(i * {bj} + j) * 16 + r] = *reinterpret_cast<const float*>(tile + row * {pitch} + col * 4);",
+                    "      }"]
+        out += ["}", ""]
+    return "\n".join(out)

@@ -1,0 +1,100 @@
+#pragma once
+// Body shared by the three matrix packages of the one-epilogue example.  HOME selects where the wave's
+// 64 x 64 fp32 accumulator is when it is handed over: 0 = accumulation registers, 1 = vector registers,
+// 2 = a row-major tile in LDS.  Everything else -- the ring protocol, the MFMA loop -- is the matrix role
+// of the three-package GEMM example.
+#include <pipelink/ring.hpp>
+#include "include/oe_abi.h"
+
+extern "C" __device__ int pipelink_gs_depth();
+extern "C" __device__ int pipelink_gs_ring();
+extern "C" __device__ int pipelink_gs_full();
+extern "C" __device__ int pipelink_gs_empty();
+extern "C" __device__ int pipelink_oe_warp_mma();
+extern "C" __device__ void pipelink_call_epilogue(const void* view, const OeTile* tile, const void* source);
+
+extern __shared__ __attribute__((aligned(1024))) unsigned char pipelink_smem[];
+
+namespace oe_mma {
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ v8bf read_frag(const unsigned char* rows, int row, int chunk) {
+  const v4i raw = *reinterpret_cast<const v4i*>(rows + row * 128 + 16 * (chunk ^ (row & 7)));
+  return __builtin_bit_cast(v8bf, raw);
+}
+
+// `tile_lds` is the wave's LDS tile for HOME 2 (unused otherwise)
+template <int HOME>
+__device__ __forceinline__ void role(const void* params, unsigned char* tile_lds) {
+  const OeMmaParams& p = *static_cast<const OeMmaParams*>(params);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) - pipelink_oe_warp_mma();
+  const int depth = pipelink_gs_depth();
+  const unsigned char* ring = pipelink_smem + pipelink_gs_ring();
+  const int tiles_n = p.n / OE_TILE;
+  const OeTile tile{(int)(blockIdx.x / tiles_n) * OE_TILE + 64 * (wave >> 1), (int)(blockIdx.x % tiles_n) * OE_TILE + 64 * (wave & 1)};
+  const int arow = 64 * (wave >> 1) + (lane & 31), brow = 64 * (wave & 1) + (lane & 31), half = lane >> 5;
+  v16f acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  const int stages = p.k / OE_TILE_K;
+  bool ok = true;
+  for (int s = 0; s < stages; ++s) {
+    const int slot = s % depth, use = s / depth;
+    ok &= pl::ring_wait(pl::ring_counter(pipelink_smem, pipelink_gs_full(), slot), (uint32_t)use + 1u);
+    const unsigned char* a_rows = ring + slot * OE_STAGE_BYTES;
+    const unsigned char* b_rows = a_rows + OE_TILE * 128;
+    v8bf a[4][2], b[4][2];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        a[kk][i] = read_frag(a_rows, arow + 32 * i, 2 * kk + half);
+        b[kk][i] = read_frag(b_rows, brow + 32 * i, 2 * kk + half);
+      }
+    pl::ring_wait_reads();
+    if (lane == 0) pl::ring_arrive(pl::ring_counter(pipelink_smem, pipelink_gs_empty(), slot));
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk][i], b[kk][j], acc[i][j], 0, 0, 0);
+  }
+  if (!ok && lane == 0) atomicOr(p.status, 2u);
+  const pipelink_host_view view{params, nullptr};
+  if constexpr (HOME == 2) {
+    // row-major fp32 tile, rows OE_LDS_PITCH bytes apart
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = 32 * i + 8 * (r / 4) + 4 * (lane >> 5) + r % 4, col = 32 * j + (lane & 31);
+          *reinterpret_cast<float*>(tile_lds + row * OE_LDS_PITCH + col * 4) = acc[i][j][r];
+        }
+    pipelink_call_epilogue(&view, &tile, tile_lds);
+  } else {
+    // the frame handed over: 64 floats per lane in fragment order, pinned in the home's register class
+    float frame[64];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float v = acc[i][j][r];
+          if constexpr (HOME == 0) asm volatile("" : "+a"(v)); else asm volatile("" : "+v"(v));
+          frame[(i * 2 + j) * 16 + r] = v;
+        }
+    pipelink_call_epilogue(&view, &tile, frame);
+  }
+}
+}  // namespace oe_mma

@@ -1,0 +1,142 @@
+"""One epilogue, many producers: a bf16 GEMM whose accumulator lives in AGPRs, in VGPRs or in an LDS tile,
+and ONE epilogue package (per-column scale + bias, bf16 out) linked against each; the linker generates the
+accumulator import for the producer's home.
+
+CPU part: the three links (routes, ring depth, the epilogue package byte for byte the same in all three),
+the rejected connections.  GPU part (marked gpu): M = N = K = 8192 -- every linked image byte-identical to
+its one-unit control and to the other homes, sampled rows against torch-CPU fp32 within the bf16 bar."""
+import json
+import shutil
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm_gelu as gg
+from pipelink_amd.pipec import linker, plink
+from pipelink_amd.pipec.clauses import PipeLinkError
+from pipelink_amd.stages.one_epilogue import build as oe_build
+
+ROOT = Path(__file__).resolve().parents[1]
+needs_rocm = pytest.mark.skipif(shutil.which("hipcc") is None and not Path("/opt/rocm/bin/hipcc").exists(),
+                                reason="needs the ROCm toolchain")
+
+
+def test_scale_bias_oracle_pins():
+    a, b, scale, bias = gg.scale_bias_inputs(64, 96, 128, seed=3)
+    full = gg.gemm_scale_bias_torch(a, b, scale, bias).float()
+    acc = a.double() @ b.double()
+    want = (acc * scale.double() + bias.double())
+    assert (full.double() - want).abs().max() <= want.abs().max() * 2.0 ** -8        # bf16 rounding of the result
+    rows = torch.tensor([5, 0, 63])
+    assert torch.equal(gg.gemm_scale_bias_torch(a, b, scale, bias, rows).float(), full[rows])
+    zero = gg.gemm_scale_bias_torch(a, b, torch.zeros_like(scale), bias).float()
+    assert torch.equal(zero, bias.to(torch.bfloat16).float().expand(64, 96))          # scale 0 leaves the bias
+    assert a.float().std().item() == pytest.approx(0.02, rel=0.05)
+
+
+@pytest.fixture(scope="module")
+def example(tmp_path_factory):
+    out = tmp_path_factory.mktemp("one_epilogue")
+    return out, oe_build.build(out=out, one_unit=False)
+
+
+@needs_rocm
+def test_one_epilogue_package_links_against_three_homes(example):
+    out, res = example
+    links = res["links"]
+    routes = {h: links[h]["tensor_plans"][0]["route"] for h in oe_build.HOMES}
+    assert routes == {"agpr": "accvgpr_receipt", "vgpr": "register_copy", "lds": "lds_load"}
+    # the same epilogue and loader packages, byte for byte, in all three links
+    assert len({links[h]["input_hashes"]["oe.epilogue"] for h in oe_build.HOMES}) == 1
+    assert len({links[h]["input_hashes"]["gs.loader"] for h in oe_build.HOMES}) == 1
+    # registers: the deepest ring fits; the LDS home claims 4 x 64 x 272 B of tiles and the ring settles for depth 2
+    assert links["agpr"]["bindings"]["pipelink_gs_depth"] == links["vgpr"]["bindings"]["pipelink_gs_depth"] == [4, "solved"]
+    assert links["lds"]["bindings"]["pipelink_gs_depth"] == [2, "solved"]
+    assert links["lds"]["dyn_smem_bytes"] == 2 * 32768 + 4 * 64 * 272 + 2 * 2 * 16 == 135232
+    assert links["agpr"]["observed"]["agpr_count"] >= 64 and links["vgpr"]["observed"]["agpr_count"] == 0
+    for h in oe_build.HOMES:
+        assert links[h]["observed"]["calls"] == 0 and links[h]["observed"]["private_segment_fixed_size"] == 0
+        stub = (out / h / "link" / "stub.hip").read_text()
+        assert "oe_epilogue_import_acc(const void* source, float* dest)" in stub and f"route {routes[h]}" in stub
+    assert "v_accvgpr_read_b32" in (out / "agpr" / "link" / "stub.hip").read_text()
+
+
+def _relink(example_dir: Path, tmp_path: Path, home: str, stage_id: str | None, mutate, pipeline_mutate=None) -> Path:
+    for f in (example_dir / home).glob("*.plink"):
+        shutil.copy(f, tmp_path / f.name)
+    pipeline = json.loads((example_dir / home / "pipeline.json").read_text())
+    if pipeline_mutate:
+        pipeline_mutate(pipeline["pipeline"])
+    (tmp_path / "pipeline.json").write_text(json.dumps(pipeline))
+    if stage_id:
+        manifest, payload = plink.read(tmp_path / f"{stage_id}.plink")
+        mutate(manifest)
+        manifest["payload"] = {"file": "stage.o"}
+        plink.pack(manifest, payload, tmp_path / f"{stage_id}.plink")
+    return tmp_path / "pipeline.json"
+
+
+@needs_rocm
+def test_rejected_tensor_connections_are_named(example, tmp_path):
+    cases = [
+        ("vgpr", "oe.mma.vgpr", lambda m: m["tensor"]["exports"][0].update(dtype="f16"), None, "T-CONTRACT",
+         "pipeline.tensor_connections.acc", "exported and imported tensor identities disagree"),
+        ("vgpr", "oe.mma.vgpr", lambda m: m["tensor"]["exports"][0].update(home="tmem"), None, "T-PLAN",
+         "pipeline.tensor_connections.acc", "no transport route reads this home and layout"),
+        ("lds", "oe.mma.lds", lambda m: m["tensor"]["exports"][0].update(row_pitch_bytes=128), None, "T-CONTRACT",
+         "pipeline.tensor_connections.acc", "row pitch of the exported tile is smaller than a row or not a multiple of 4"),
+        ("agpr", None, None, lambda p: p.update(tensor_connections=[]), "T-CONTRACT",
+         "stages.oe.epilogue.tensor.imports.acc", "import is not fed by any tensor connection"),
+        ("agpr", None, None, lambda p: p["tensor_connections"][0].update(export="accumulator"), "T-CONTRACT",
+         "pipeline.tensor_connections.acc", "connection names an export or import its stage does not declare"),
+    ]
+    for i, (home, sid, mutate, pmutate, clause, path, message) in enumerate(cases):
+        sub = tmp_path / str(i)
+        sub.mkdir()
+        with pytest.raises(PipeLinkError) as err:
+            linker.link(_relink(example[0], sub, home, sid, mutate, pmutate), sub / "link", codegen=False)
+        first = err.value.failures[0]
+        assert (first.clause_id, first.path, first.message) == (clause, path, message), str(err.value)
+
+
+# ---- GPU ---------------------------------------------------------------------------------------------------
+
+def _bits(t: torch.Tensor) -> np.ndarray:
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("size", [512, 8192])
+def test_three_homes_one_epilogue_bit_exact_and_within_the_bf16_bar(size):
+    from pipelink_amd.host.one_epilogue import open_session
+
+    a, b, scale, bias = gg.scale_bias_inputs(size, size, size, seed=0)
+    a_bits, bt_bits = _bits(a), _bits(b.t())
+    results = {}
+    for home in oe_build.HOMES:
+        paths = oe_build.images(home)
+        sess = open_session(paths["link_json"], home, a_bits, bt_bits, bias.numpy(), scale.numpy())
+        try:
+            print(f"home {home} size {size}", flush=True)
+            sess.launch()
+            sess.synchronize()
+            assert sess.read("status")[0] == 0, "a ring wait gave up"
+            results[home] = sess.read("c")
+            control = sess.with_image(paths["one_unit"])
+            sess.write("c", np.full((size, size), 0x7FC0, dtype=np.uint16))    # bf16 NaN
+            control.launch()
+            control.synchronize()
+            assert sess.read("status")[0] == 0
+            assert np.array_equal(sess.read("c"), results[home]), f"{home}: linked and one-unit images differ"
+        finally:
+            sess.close()
+    assert np.array_equal(results["agpr"], results["vgpr"]) and np.array_equal(results["agpr"], results["lds"])
+    rows = torch.arange(size) if size <= 512 else torch.from_numpy(np.random.default_rng(0).choice(size, 48, replace=False))
+    want = gg.gemm_scale_bias_torch(a, b, scale, bias, rows).float().numpy()
+    got = torch.from_numpy(results["agpr"].view(np.int16)).view(torch.bfloat16).float().numpy()[rows.numpy()]
+    assert np.isfinite(got).all()
+    rel = np.abs(got - want) / np.maximum(np.abs(want), 2.0 ** -6)   # results are O(0.1); a floor for the few near zero
+    assert rel.max() <= 1e-2
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 3e-3
