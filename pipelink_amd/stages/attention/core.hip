@@ -1,0 +1,220 @@
+// Package fa.core: flash-attention forward for one tile of 128 queries of one head.
+//
+// Orientation.  Scores are computed transposed, S^T = K . Q^T (keys are the MFMA rows, queries the
+// columns), so that a lane holds ONE query (column lane % 32) and 16 of the block's 32 keys: row maxima
+// and sums are in-register reductions plus one exchange between lane l and l ^ 32.  The probabilities
+// are then, register for register, the B operand of O^T += V^T . P^T -- the contraction index of an MFMA
+// is only a summation order, and V^T is read from LDS in the order the registers hold the keys:
+//   group g of 16 keys (registers 8g .. 8g+7 of a 32-key score tile), lane half h = lane / 32:
+//   elements 0-3 = keys 16g + 4h + 0..3, elements 4-7 = keys 16g + 8 + 4h + 0..3.
+// V arrives row-major [key][d]; a thread loads 8 consecutive d of one key and writes them into the
+// transposed LDS tile V^T[d][key] (2-byte writes), so that the A operand of the second product is two
+// 8-byte reads.  K is the A operand of the first product as stored (row-major), and goes global -> LDS
+// directly, 16-byte chunks swizzled by position = chunk ^ (key % 16).
+//
+// Two LDS buffers per operand: block i + 1 is in flight while block i is multiplied; one barrier per block.
+#include <pipelink/stage.hpp>
+#ifndef PIPELINK_EMIT
+#include <hip/hip_runtime.h>
+#include "include/fa_abi.h"
+
+extern "C" __device__ int pipelink_fa_kv();  // byte offset of the K / V^T buffers in dynamic LDS
+extern "C" __device__ int pipelink_call_mask_key_count(const void* view, int q_first, int q_last);
+extern "C" __device__ int pipelink_call_mask_all_visible(const void* view, int q_first, int q_last, int k_first, int k_last);
+extern "C" __device__ int pipelink_call_mask_visible(const void* view, int q, int k);
+
+extern __shared__ __attribute__((aligned(1024))) unsigned char pipelink_smem[];
+
+namespace fa_core {
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v8f __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+constexpr int K_BYTES = FA_K_BLOCK * FA_D * 2;     // 16 KB: [64 keys][256 bytes]
+constexpr int VT_PITCH = FA_K_BLOCK * 2 + 8;       // bytes between d rows of V^T[128 d][64 keys]
+constexpr int VT_BYTES = FA_D * VT_PITCH;          // 17 KB
+constexpr int BUF_BYTES = K_BYTES + VT_BYTES;
+constexpr float MASKED = -1.0e30f;
+
+// K block -> LDS: 64 keys x 256 B; one load instruction of a wave moves 4 keys (1 KB)
+__device__ __forceinline__ void issue_k(__amdgpu_buffer_rsrc_t k, uint32_t first_key_byte, unsigned char* dst, int wave, int lane) {
+  const int kr = lane >> 4, pos = lane & 15;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int key = (wave * 4 + j) * 4 + kr;  // 0..63
+    const uint32_t off = first_key_byte + (uint32_t)key * (FA_D * 2) + 16u * (uint32_t)(pos ^ (key & 15));
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(k, (lds_ptr)(dst + (wave * 4 + j) * 1024), 16, (int)off, 0, 0, 0);
+  }
+}
+// V block -> registers: thread t loads, for j = 0..3, 8 consecutive d (chunk t % 16) of key t / 16 + 16 j
+__device__ __forceinline__ void load_v(__amdgpu_buffer_rsrc_t v, uint32_t first_key_byte, int tid, v4i (&regs)[4]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int key = (tid >> 4) + 16 * j;
+    regs[j] = __builtin_amdgcn_raw_buffer_load_b128(v, (int)(first_key_byte + (uint32_t)key * (FA_D * 2) + 16u * (uint32_t)(tid & 15)), 0, 0);
+  }
+}
+__device__ __forceinline__ void store_vt(unsigned char* vt, int tid, const v4i (&regs)[4]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int key = (tid >> 4) + 16 * j, d0 = 8 * (tid & 15);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t word = (uint32_t)regs[j][e >> 1];
+      *reinterpret_cast<uint16_t*>(vt + (d0 + e) * VT_PITCH + key * 2) = (uint16_t)((e & 1) ? word >> 16 : word);
+    }
+  }
+}
+}  // namespace fa_core
+
+extern "C" __device__ void fa_core_role_core(const void* params, unsigned variant) {
+  (void)variant;
+  using namespace fa_core;
+  const FaCoreParams& p = *static_cast<const FaCoreParams*>(params);
+  const pipelink_host_view view{params, nullptr};
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5, l32 = lane & 31;
+  const int q_tiles = p.seq / FA_Q_TILE;
+  const int tile = blockIdx.x % q_tiles, bh = blockIdx.x / q_tiles;  // bh = batch * q_heads + head
+  const int b = bh / p.q_heads, h = bh % p.q_heads, kvh = h / (p.q_heads / p.kv_heads);
+  const int q0 = tile * FA_Q_TILE, qw = q0 + 32 * wave;               // the wave's first query
+  const uint32_t head_bytes = (uint32_t)p.seq * FA_D * 2;
+  const __amdgpu_buffer_rsrc_t kres = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(p.k) + ((int64_t)b * p.kv_heads + kvh) * p.seq * FA_D, 0, (int)head_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t vres = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(p.v) + ((int64_t)b * p.kv_heads + kvh) * p.seq * FA_D, 0, (int)head_bytes, 0x00020000);
+  unsigned char* buf = pipelink_smem + pipelink_fa_kv();
+
+  // this lane's query row as the B operand of S^T = K . Q^T: 16 bytes per 16-element step of d
+  v8bf qf[8];
+  {
+    const uint16_t* qrow = p.q + (((int64_t)b * p.q_heads + h) * p.seq + qw + l32) * FA_D;
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) qf[kk] = __builtin_bit_cast(v8bf, *reinterpret_cast<const v4i*>(qrow + 16 * kk + 8 * half));
+  }
+  v16f o[4];  // O^T: [d block][16 d of the block] for this lane's query
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[db][r] = 0.0f;
+  float row_max = MASKED, row_sum = 0.0f;
+
+  const int keys = pipelink_call_mask_key_count(&view, q0, q0 + FA_Q_TILE - 1);
+  const int blocks = (keys + FA_K_BLOCK - 1) / FA_K_BLOCK;
+  const int wave_keys = pipelink_call_mask_key_count(&view, qw, qw + 31);
+  v4i vregs[4];
+  issue_k(kres, 0u, buf, wave, lane);
+  load_v(vres, 0u, tid, vregs);
+  for (int i = 0; i < blocks; ++i) {
+    unsigned char* kbuf = buf + (i & 1) * BUF_BYTES;
+    unsigned char* vt = kbuf + K_BYTES;
+    store_vt(vt, tid, vregs);  // waits for the V loads of block i
+    __syncthreads();           // K block i has landed (the barrier drains this wave's loads), V^T block i is written
+    if (i + 1 < blocks) {
+      issue_k(kres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + ((i + 1) & 1) * BUF_BYTES, wave, lane);
+      load_v(vres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, tid, vregs);
+    }
+    const int k0 = i * FA_K_BLOCK;
+    if (k0 >= wave_keys) continue;  // no query of this wave sees a key this far on: only the loads and the barrier
+    // ---- S^T = K . Q^T : two 32-key tiles -----------------------------------------------------------
+    v16f s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[t][r] = 0.0f;
+      const int key = 32 * t + l32;
+#pragma unroll
+      for (int kk = 0; kk < 8; ++kk) {
+        const v4i raw = *reinterpret_cast<const v4i*>(kbuf + key * (FA_D * 2) + 16 * ((2 * kk + half) ^ (key & 15)));
+        s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, raw), qf[kk], s[t], 0, 0, 0);
+      }
+    }
+    // ---- mask, online softmax ------------------------------------------------------------------------
+    const int query = qw + l32;
+    const bool all = pipelink_call_mask_all_visible(&view, qw, qw + 31, k0, k0 + FA_K_BLOCK - 1);
+    float block_max = MASKED;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = k0 + 32 * t + 8 * (r / 4) + 4 * half + r % 4;
+        float x = s[t][r] * p.scale_log2e;
+        if (!all && !pipelink_call_mask_visible(&view, query, key)) x = MASKED;
+        s[t][r] = x;
+        block_max = fmaxf(block_max, x);
+      }
+    block_max = fmaxf(block_max, __shfl_xor(block_max, 32));
+    const float new_max = fmaxf(row_max, block_max);
+    const float alpha = __builtin_amdgcn_exp2f(row_max - new_max);
+    row_max = new_max;
+    float block_sum = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float e = s[t][r] <= 0.5f * MASKED ? 0.0f : __builtin_amdgcn_exp2f(s[t][r] - new_max);
+        s[t][r] = e;
+        block_sum += e;
+      }
+    block_sum += __shfl_xor(block_sum, 32);
+    row_sum = row_sum * alpha + block_sum;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+    // ---- O^T += V^T . P^T : four groups of 16 keys, four 32-row blocks of d ----------------------------
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        v8f pf;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pf[e] = s[t][8 * g + e];
+        const v8bf pb = __builtin_convertvector(pf, v8bf);
+        const int kcol = 2 * (32 * t + 16 * g + 4 * half);  // byte offset of the lane's first key in a V^T row
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          const unsigned char* row = vt + (32 * db + l32) * VT_PITCH + kcol;
+          const v2i lo = *reinterpret_cast<const v2i*>(row), hi = *reinterpret_cast<const v2i*>(row + 16);
+          const v4i raw = {lo.x, lo.y, hi.x, hi.y};
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, raw), pb, o[db], 0, 0, 0);
+        }
+      }
+  }
+  // ---- O[b][query][h][d] = O^T / row_sum, bf16 ------------------------------------------------------------
+  const float inv = row_sum > 0.0f ? __builtin_amdgcn_rcpf(row_sum) : 0.0f;
+  uint16_t* orow = p.o + ((int64_t)b * p.seq + qw + l32) * ((int64_t)p.q_heads * FA_D) + (int64_t)h * FA_D;
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      const v4f f = {o[db][4 * q4] * inv, o[db][4 * q4 + 1] * inv, o[db][4 * q4 + 2] * inv, o[db][4 * q4 + 3] * inv};
+      const v4bf packed = __builtin_convertvector(f, v4bf);
+      *reinterpret_cast<v2i*>(orow + 32 * db + 8 * q4 + 4 * half) = __builtin_bit_cast(v2i, packed);
+    }
+}
+#else
+#include "include/fa_abi.h"
+#endif
+
+PL_STAGE("fa.core", "0.1.0");
+PL_PARAMS(FaCoreParams);
+PL_ROLE(core, fa_core_role_core, 4);
+PL_TOPOLOGY(false, "static");
+PL_VARIANT(0, {});
+PL_CALL(mask_key_count, "mask_key_count",
+        "extern \"C\" __device__ int pipelink_call_mask_key_count(const void* view, int q_first, int q_last);");
+PL_CALL(mask_all_visible, "mask_all_visible",
+        "extern \"C\" __device__ int pipelink_call_mask_all_visible(const void* view, int q_first, int q_last, int k_first, int k_last);");
+PL_CALL(mask_visible, "mask_visible",
+        "extern \"C\" __device__ int pipelink_call_mask_visible(const void* view, int q, int k);");
+// two buffers of (K block 16 KB + V^T block 17 KB)
+PL_CLAIM("pipelink_fa_kv", "smem", 2 * (64 * 128 * 2 + 128 * (64 * 2 + 8)), 1024, "kernel");
+PL_USES("pipelink_fa_kv");
+PL_PRELUDE("include/fa_abi.h");
+PL_EMIT_MAIN()
