@@ -27,7 +27,7 @@ from typing import Any
 from . import plink
 from .channels import expand_all, pair_channels
 from .clauses import ClauseFailure, LinkError, PipeLinkError
-from .glue import KERNEL_SYMBOL, collect_preludes, generate_dispatch, generate_stub, params_layout
+from .glue import waves_per_simd, KERNEL_SYMBOL, collect_preludes, generate_dispatch, generate_stub, params_layout
 from .manifest import Pipeline, Stage, load_pipeline, load_stage_manifest, validate_assembly
 from .pack import DEVICE_FLAGS, HIPCC, INCLUDE_DIR, LLVM_BIN
 from .tensors import generate_adapters, plan_connections
@@ -166,7 +166,8 @@ def link(pipeline_path: str | Path, out_dir: str | Path, *, include_dirs: list[s
         if observed["calls"]:
             _fail("L-LINK", "observed.calls", "linked kernel still calls across a package seam: an export was not inlined",
                   **observed)
-        if observed["vgpr_count"] > solution.regs_cap:
+        regs_cap = min(solution.regs_cap, pipeline.profile.regs_per_lane // waves_per_simd(stages))
+        if observed["vgpr_count"] > regs_cap:
             _fail("L-REGS", "observed.vgpr_count", "linked kernel needs more registers than the launch leaves per lane",
                   **observed)
     result = {

@@ -7,10 +7,13 @@
 // is only a summation order, and V^T is read from LDS in the order the registers hold the keys:
 //   group g of 16 keys (registers 8g .. 8g+7 of a 32-key score tile), lane half h = lane / 32:
 //   elements 0-3 = keys 16g + 4h + 0..3, elements 4-7 = keys 16g + 8 + 4h + 0..3.
-// V arrives row-major [key][d]; a thread loads 8 consecutive d of one key and writes them into the
-// transposed LDS tile V^T[d][key] (2-byte writes), so that the A operand of the second product is two
-// 8-byte reads.  K is the A operand of the first product as stored (row-major), and goes global -> LDS
-// directly, 16-byte chunks swizzled by position = chunk ^ (key % 16).
+// K and V both go global -> LDS as stored (row-major [key][d], 16-byte chunks swizzled by position =
+// chunk ^ (key % 16)).  K rows are the A operand of the first product as they are.  The A operand of the
+// second product wants, per lane, four consecutive KEYS at one d -- a column of the V tile: that is what
+// ds_read_b64_tr_b16 delivers.  In a group of 16 lanes, lane i hands in the address of 4 consecutive d
+// (8 bytes) and lane j receives element j % 4 of the data of lanes j / 4, j / 4 + 4, j / 4 + 8, j / 4 + 12
+// (measured with a probe); so lane i points at key kbase + i / 4, d = dbase + 4 (i % 4), and lane j gets keys
+// kbase .. kbase + 3 at d = dbase + j.
 //
 // Two LDS buffers per operand: block i + 1 is in flight while block i is multiplied; one barrier per block.
 #include <pipelink/stage.hpp>
@@ -35,40 +38,26 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
-constexpr int K_BYTES = FA_K_BLOCK * FA_D * 2;     // 16 KB: [64 keys][256 bytes]
-constexpr int VT_PITCH = FA_K_BLOCK * 2 + 8;       // bytes between d rows of V^T[128 d][64 keys]
-constexpr int VT_BYTES = FA_D * VT_PITCH;          // 17 KB
-constexpr int BUF_BYTES = K_BYTES + VT_BYTES;
+constexpr int K_BYTES = FA_K_BLOCK * FA_D * 2;     // 16 KB: [64 keys][256 bytes], the same for V
+constexpr int BUF_BYTES = 2 * K_BYTES;
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4s* lds_v4s;
 constexpr float MASKED = -1.0e30f;
 
-// K block -> LDS: 64 keys x 256 B; one load instruction of a wave moves 4 keys (1 KB)
-__device__ __forceinline__ void issue_k(__amdgpu_buffer_rsrc_t k, uint32_t first_key_byte, unsigned char* dst, int wave, int lane) {
+// one 64-key block of K or V -> LDS: 64 keys x 256 B; one load instruction of a wave moves 4 keys (1 KB)
+__device__ __forceinline__ void issue_block(__amdgpu_buffer_rsrc_t src, uint32_t first_key_byte, unsigned char* dst, int wave, int lane) {
   const int kr = lane >> 4, pos = lane & 15;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int key = (wave * 4 + j) * 4 + kr;  // 0..63
     const uint32_t off = first_key_byte + (uint32_t)key * (FA_D * 2) + 16u * (uint32_t)(pos ^ (key & 15));
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(k, (lds_ptr)(dst + (wave * 4 + j) * 1024), 16, (int)off, 0, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (lds_ptr)(dst + (wave * 4 + j) * 1024), 16, (int)off, 0, 0, 0);
   }
 }
-// V block -> registers: thread t loads, for j = 0..3, 8 consecutive d (chunk t % 16) of key t / 16 + 16 j
-__device__ __forceinline__ void load_v(__amdgpu_buffer_rsrc_t v, uint32_t first_key_byte, int tid, v4i (&regs)[4]) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int key = (tid >> 4) + 16 * j;
-    regs[j] = __builtin_amdgcn_raw_buffer_load_b128(v, (int)(first_key_byte + (uint32_t)key * (FA_D * 2) + 16u * (uint32_t)(tid & 15)), 0, 0);
-  }
-}
-__device__ __forceinline__ void store_vt(unsigned char* vt, int tid, const v4i (&regs)[4]) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int key = (tid >> 4) + 16 * j, d0 = 8 * (tid & 15);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const uint32_t word = (uint32_t)regs[j][e >> 1];
-      *reinterpret_cast<uint16_t*>(vt + (d0 + e) * VT_PITCH + key * 2) = (uint16_t)((e & 1) ? word >> 16 : word);
-    }
-  }
+// 4 consecutive keys from `key` on, at the d this lane's group position stands for (see the head of the file)
+__device__ __forceinline__ v4s read_v_column(const unsigned char* vbuf, int key, int d) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (lds_v4s)(const_cast<unsigned char*>(vbuf) + key * (FA_D * 2) + 16 * ((d >> 3) ^ (key & 15)) + 2 * (d & 4)));
 }
 }  // namespace fa_core
 
@@ -80,7 +69,10 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, l32 = lane & 31;
   const int q_tiles = p.seq / FA_Q_TILE;
-  const int tile = blockIdx.x % q_tiles, bh = blockIdx.x / q_tiles;  // bh = batch * q_heads + head
+  // Causal tiles cost in proportion to their position: the latest (longest) tiles of every head are
+  // dispatched first, so that the grid does not end on a few long ones.  bh = batch * q_heads + head.
+  const int heads = p.batch * p.q_heads;
+  const int tile = q_tiles - 1 - (int)(blockIdx.x / heads), bh = blockIdx.x % heads;
   const int b = bh / p.q_heads, h = bh % p.q_heads, kvh = h / (p.q_heads / p.kv_heads);
   const int q0 = tile * FA_Q_TILE, qw = q0 + 32 * wave;               // the wave's first query
   const uint32_t head_bytes = (uint32_t)p.seq * FA_D * 2;
@@ -107,17 +99,16 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
   const int keys = pipelink_call_mask_key_count(&view, q0, q0 + FA_Q_TILE - 1);
   const int blocks = (keys + FA_K_BLOCK - 1) / FA_K_BLOCK;
   const int wave_keys = pipelink_call_mask_key_count(&view, qw, qw + 31);
-  v4i vregs[4];
-  issue_k(kres, 0u, buf, wave, lane);
-  load_v(vres, 0u, tid, vregs);
+  issue_block(kres, 0u, buf, wave, lane);
+  issue_block(vres, 0u, buf + K_BYTES, wave, lane);
+  const int li = lane & 15, dgroup = 16 * ((lane >> 4) & 1);  // position in the 16-lane group, the group's first d in a 32-row block
   for (int i = 0; i < blocks; ++i) {
     unsigned char* kbuf = buf + (i & 1) * BUF_BYTES;
-    unsigned char* vt = kbuf + K_BYTES;
-    store_vt(vt, tid, vregs);  // waits for the V loads of block i
-    __syncthreads();           // K block i has landed (the barrier drains this wave's loads), V^T block i is written
+    const unsigned char* vbuf = kbuf + K_BYTES;
+    __syncthreads();  // blocks i of K and V have landed (the barrier drains every wave's loads); buffers of block i - 1 are free
     if (i + 1 < blocks) {
-      issue_k(kres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + ((i + 1) & 1) * BUF_BYTES, wave, lane);
-      load_v(vres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, tid, vregs);
+      issue_block(kres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + ((i + 1) & 1) * BUF_BYTES, wave, lane);
+      issue_block(vres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + ((i + 1) & 1) * BUF_BYTES + K_BYTES, wave, lane);
     }
     const int k0 = i * FA_K_BLOCK;
     if (k0 >= wave_keys) continue;  // no query of this wave sees a key this far on: only the loads and the barrier
@@ -176,12 +167,13 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
 #pragma unroll
         for (int e = 0; e < 8; ++e) pf[e] = s[t][8 * g + e];
         const v8bf pb = __builtin_convertvector(pf, v8bf);
-        const int kcol = 2 * (32 * t + 16 * g + 4 * half);  // byte offset of the lane's first key in a V^T row
+        const int key = 32 * t + 16 * g + 4 * half + (li >> 2);  // the row this lane points at: its group's first key + li / 4
 #pragma unroll
         for (int db = 0; db < 4; ++db) {
-          const unsigned char* row = vt + (32 * db + l32) * VT_PITCH + kcol;
-          const v2i lo = *reinterpret_cast<const v2i*>(row), hi = *reinterpret_cast<const v2i*>(row + 16);
-          const v4i raw = {lo.x, lo.y, hi.x, hi.y};
+          const int d = 32 * db + dgroup + 4 * (li & 3);
+          const v4s lo = read_v_column(vbuf, key, d), hi = read_v_column(vbuf, key + 8, d);
+          const v2i lo2 = __builtin_bit_cast(v2i, lo), hi2 = __builtin_bit_cast(v2i, hi);
+          const v4i raw = {lo2.x, lo2.y, hi2.x, hi2.y};
           o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, raw), pb, o[db], 0, 0, 0);
         }
       }
@@ -213,8 +205,11 @@ PL_CALL(mask_all_visible, "mask_all_visible",
         "extern \"C\" __device__ int pipelink_call_mask_all_visible(const void* view, int q_first, int q_last, int k_first, int k_last);");
 PL_CALL(mask_visible, "mask_visible",
         "extern \"C\" __device__ int pipelink_call_mask_visible(const void* view, int q, int k);");
-// two buffers of (K block 16 KB + V^T block 17 KB)
-PL_CLAIM("pipelink_fa_kv", "smem", 2 * (64 * 128 * 2 + 128 * (64 * 2 + 8)), 1024, "kernel");
+// two buffers of (K block 16 KB + V block 16 KB)
+PL_CLAIM("pipelink_fa_kv", "smem", 2 * 2 * (64 * 128 * 2), 1024, "kernel");
 PL_USES("pipelink_fa_kv");
+// two workgroups per CU (two waves per SIMD, 256 registers per lane each): one multiplies while the other
+// is in its softmax or waits at its barrier; 2 x 67.6 KB of LDS fit
+PL_FACT("launch.waves_per_simd", 2);
 PL_PRELUDE("include/fa_abi.h");
 PL_EMIT_MAIN()

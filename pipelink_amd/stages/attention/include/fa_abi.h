@@ -2,8 +2,8 @@
  * head, bf16 in, fp32 accumulate, bf16 out, grouped-query (several query heads share a KV head).
  *
  *   fa.core         role `core`, 4 waves: one workgroup owns 128 consecutive queries of one query head;
- *                   a wave owns 32 of them.  Streams 64-key blocks of K (row-major, via LDS) and V
- *                   (transposed on its way into LDS), online softmax in registers, MFMA 32x32x16 bf16.
+ *                   a wave owns 32 of them.  Streams 64-key blocks of K and V through LDS (V read
+ *                   column-wise with the transposing LDS read), online softmax in registers, MFMA 32x32x16 bf16.
  *   fa.mask.causal  exports that say which keys a query may see; the core calls them through call
  *                   channels, so another mask is another package (campaigns/attention/src/sm90 in the
  *                   reference: stage_core.cu, stage_mask_default.cu / stage_mask_window.cu).

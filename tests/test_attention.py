@@ -46,7 +46,7 @@ def test_link_records_core_and_mask_packages(example):
     link = res["link"]
     assert [e["stage_id"] for e in link["params"]["entries"]] == ["fa.core", "fa.mask.causal"]
     assert [(e["offset"], e["bytes"]) for e in link["params"]["entries"]] == [(0, 56), (56, 8)]
-    assert link["threads"] == 256 and link["dyn_smem_bytes"] == 2 * (64 * 256 + 128 * 136) == 67584
+    assert link["threads"] == 256 and link["dyn_smem_bytes"] == 2 * 2 * 64 * 256 == 65536
     assert {e["channel"] for e in link["protocol_expansions"]} == {"mask_key_count", "mask_all_visible", "mask_visible"}
     obs = link["observed"]
     assert obs["calls"] == 0 and obs["mfma"] == 32 and obs["private_segment_fixed_size"] == 0   # the mask is inlined
