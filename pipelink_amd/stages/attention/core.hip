@@ -125,22 +125,27 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
         s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, raw), qf[kk], s[t], 0, 0, 0);
       }
     }
-    // ---- mask, online softmax ------------------------------------------------------------------------
+    // ---- mask, online softmax (in units of log2: exp2(x * scale_log2e - max)) -------------------------------
     const int query = qw + l32;
     const bool all = pipelink_call_mask_all_visible(&view, qw, qw + 31, k0, k0 + FA_K_BLOCK - 1);
+    if (!all) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = k0 + 32 * t + 8 * (r / 4) + 4 * half + r % 4;
+          if (!pipelink_call_mask_visible(&view, query, key)) s[t][r] = MASKED;
+        }
+    }
     float block_max = MASKED;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = k0 + 32 * t + 8 * (r / 4) + 4 * half + r % 4;
-        float x = s[t][r] * p.scale_log2e;
-        if (!all && !pipelink_call_mask_visible(&view, query, key)) x = MASKED;
-        s[t][r] = x;
-        block_max = fmaxf(block_max, x);
-      }
+      for (int r = 0; r < 16; ++r) block_max = fmaxf(block_max, s[t][r]);
     block_max = fmaxf(block_max, __shfl_xor(block_max, 32));
-    const float new_max = fmaxf(row_max, block_max);
+    // every query sees key 0, and block 0 comes first: from then on the maximum is a real score, and a
+    // masked entry (-1e30) turns into exp2(-huge) = 0 by itself
+    const float new_max = fmaxf(row_max, block_max * p.scale_log2e);
     const float alpha = __builtin_amdgcn_exp2f(row_max - new_max);
     row_max = new_max;
     float block_sum = 0.0f;
@@ -148,16 +153,18 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float e = s[t][r] <= 0.5f * MASKED ? 0.0f : __builtin_amdgcn_exp2f(s[t][r] - new_max);
+        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], p.scale_log2e, -new_max));
         s[t][r] = e;
         block_sum += e;
       }
     block_sum += __shfl_xor(block_sum, 32);
     row_sum = row_sum * alpha + block_sum;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {  // once the maxima have settled nothing needs rescaling
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+      for (int db = 0; db < 4; ++db)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+        for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+    }
     // ---- O^T += V^T . P^T : four groups of 16 keys, four 32-row blocks of d ----------------------------
 #pragma unroll
     for (int t = 0; t < 2; ++t)
