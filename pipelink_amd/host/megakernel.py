@@ -1,0 +1,33 @@
+"""Host side of the decode megakernel example on the host-less route: one launch = one decoded token."""
+from __future__ import annotations
+
+from pathlib import Path
+
+import numpy as np
+
+from ..pipec.launcher import HostlessSession, open_hostless
+from ..stages.megakernel import params as mk
+
+
+def open_session(link_json: str | Path, weights: np.ndarray, kv_cache: np.ndarray, x: np.ndarray, *, layers: int, d: int, hq: int,
+                 hkv: int, dff: int, vocab: int, pos: int, workgroups: int, backend=None, image: str | Path | None = None) -> HostlessSession:
+    """weights: packed bf16 bit patterns (uint16, see mk_abi.h); kv_cache [L, 2, smax, hkv, 64] uint16 with positions
+    0 .. pos-1 filled; x [d] float32.  `workgroups` must be a multiple of hq (each workgroup takes one
+    (head, context chunk) of the attention) and no more than can be resident at once (one per CU is safe)."""
+    smax = kv_cache.shape[2]
+    if kv_cache.shape != (layers, 2, smax, hkv, mk.HEAD_DIM) or kv_cache.dtype != np.uint16 or weights.dtype != np.uint16:
+        raise ValueError("kv_cache is [L, 2, smax, hkv, 64] uint16, weights uint16")
+    if weights.size != layers * mk.layer_elems(d, hq, hkv, dff) + d + vocab * d:
+        raise ValueError("weights do not have the packed size for these dimensions")
+    if d % 512 or dff % 512 or (hq * mk.HEAD_DIM) % 512 or hq % hkv or workgroups % hq or pos >= smax or d + 64 > 8192 or dff > 8192:
+        raise ValueError("d, dff and hq*64 must be multiples of 512 (dff <= 8192), hq a multiple of hkv, workgroups a multiple of hq, pos < smax")
+    chunks = workgroups // hq
+    if (pos + 1 + chunks - 1) // chunks > 8192 - 512:
+        raise ValueError("a context chunk does not fit the workgroup's LDS vector: use more workgroups")
+    prog = mk.program(layers)
+    buffers = {"weights": weights, "kv_cache": kv_cache, "x": x.astype(np.float32), "rope": mk.rope_table(pos), "program": prog,
+               "qkv": (((hq + 2 * hkv) * mk.HEAD_DIM,), np.float32), "attn_partial": ((hq * chunks * (mk.HEAD_DIM + 2),), np.float32),
+               "h": ((dff,), np.float32), "logits": ((vocab,), np.float32), "sync": ((4,), np.uint32)}
+    blob = lambda addr: {"mk.interp": mk.params_blob(addr, num_instr=len(prog), layers=layers, d=d, hq=hq, hkv=hkv, dff=dff,
+                                                     vocab=vocab, pos=pos, smax=smax, chunks=chunks)}
+    return open_hostless(link_json, buffers=buffers, params=blob, grid=(workgroups,), backend=backend, image=image)

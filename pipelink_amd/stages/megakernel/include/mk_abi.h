@@ -1,0 +1,67 @@
+/* Shared declarations of the decode megakernel example: one persistent kernel runs a whole decoding
+ * step of a Llama-shaped model (RMSNorm, fused QKV matvec, RoPE, attention over the KV cache, output
+ * projection, gate/up matvec + SwiGLU, down matvec, LM head) for one token.
+ *
+ * Packages (campaigns/megakernel/port/src in the reference: interpreter.cu + ops/*.cu wrapped as opcode
+ * slots): mk.interp -- the persistent role: every workgroup walks the same instruction stream, calls the
+ * op an instruction names through a call channel with its share of the work, and meets the others at a
+ * grid barrier where an instruction asks for one -- and eight op packages: mk.rmsnorm, mk.qkv, mk.rope,
+ * mk.attn, mk.oproj, mk.upgate, mk.down, mk.lmhead.  Swapping the attention package (mk.attn for
+ * mk.attn.wide) and relinking changes nothing else.
+ *
+ * Everything an op needs is in MkModel, the interpreter's params; ops have no params of their own and
+ * receive the interpreter's view. */
+#ifndef PIPELINK_MK_ABI_H
+#define PIPELINK_MK_ABI_H
+
+#include <stdint.h>
+#include <pipelink/host_view.h>
+
+#define MK_THREADS 256
+#define MK_HEAD_DIM 64
+
+enum {
+  MK_OP_RMSNORM_ATTN = 1, /* x * rsqrt(mean x^2 + eps) * attn_norm[layer]  -> LDS vector */
+  MK_OP_QKV = 2,          /* qkv = Wqkv[layer] . vector */
+  MK_OP_ATTN = 3,         /* RoPE, append to the cache, partial attention of (head, chunk) */
+  MK_OP_OPROJ = 4,        /* combine the partials; x += Wo[layer] . attention */
+  MK_OP_RMSNORM_FFN = 5,
+  MK_OP_UPGATE = 6,       /* h = silu(Wgate . vector) * (Wup . vector) */
+  MK_OP_DOWN = 7,         /* x += Wdown . h */
+  MK_OP_RMSNORM_FINAL = 8,
+  MK_OP_LMHEAD = 9        /* logits = Wlm . vector */
+};
+
+/* one instruction: 4 x int32 */
+typedef struct MkInstr {
+  int32_t opcode, layer, barrier_after, reserved;
+} MkInstr;
+
+typedef struct MkModel {
+  const uint16_t* weights; /* bf16; per layer: attn_norm[D], wqkv[(HQ+2HKV)*64][D], wo[D][HQ*64], ffn_norm[D], wgate[DFF][D],
+                              wup[DFF][D], wdown[D][DFF]; then final_norm[D], lm_head[V][D] */
+  uint16_t* kv_cache;      /* bf16 [L][2][SMAX][HKV][64] */
+  float* x;                /* [D] residual stream, in and out */
+  float* qkv;              /* [(HQ + 2 HKV) * 64] */
+  float* attn_partial;     /* [HQ][chunks][64 + 2]: unnormalised output, running maximum (log2 units), sum */
+  float* h;                /* [DFF] */
+  float* logits;           /* [V] */
+  const float* rope;       /* [2][32]: cos, sin of pos * theta^(-2 i / 64) */
+  const MkInstr* program;
+  uint32_t* sync;          /* [0] grid barrier counter (zero at launch; the kernel leaves it zero), [1] status (non-zero: a
+                              wait gave up), [2] count of workgroups that have finished (zero at launch, left zero) */
+  int32_t num_instr, layers, d, hq, hkv, dff, vocab, pos, smax, chunks;
+  float eps, attn_scale_log2e;
+} MkModel;
+
+#ifdef __cplusplus
+#ifdef __HIPCC__
+__host__ __device__
+#endif
+static inline int64_t mk_layer_elems(const MkModel* m) {
+  const int64_t d = m->d, qkv = (int64_t)(m->hq + 2 * m->hkv) * MK_HEAD_DIM;
+  return d + qkv * d + d * (int64_t)m->hq * MK_HEAD_DIM + d + 2 * (int64_t)m->dff * d + d * (int64_t)m->dff;
+}
+#endif
+
+#endif

@@ -1,0 +1,40 @@
+// Package mk.lmhead: logits = Wlm . vector for this workgroup's share of the vocabulary rows.
+#include <pipelink/stage.hpp>
+#ifndef PIPELINK_EMIT
+#include "mk_device.hpp"
+
+extern "C" __device__ void mk_lmhead_op(const void* view, const MkInstr* instr) {
+  (void)instr;
+  const MkModel& m = mk::model(view);
+  const uint16_t* w = mk::lm_head(m);
+  const float* x = mk::vec();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int first, last;
+  mk::my_rows(m.vocab, first, last);
+  int r = first + 2 * wave;
+  for (; r + 1 < last; r += 8) {
+    float a, b;
+    mk::row_dot2(w + (int64_t)r * m.d, w + (int64_t)(r + 1) * m.d, x, m.d, lane, a, b);
+    if (lane == 0) {
+      m.logits[r] = a;
+      m.logits[r + 1] = b;
+    }
+  }
+  if (r < last) {
+    const float a = mk::row_dot(w + (int64_t)r * m.d, x, m.d, lane);
+    if (lane == 0) m.logits[r] = a;
+  }
+}
+#else
+#include "include/mk_abi.h"
+#endif
+
+PL_STAGE("mk.lmhead", "0.1.0");
+PL_NO_PARAMS();
+PL_TOPOLOGY(true, "static");
+PL_VARIANT(0, {});
+PL_EXPORT(op_lmhead, mk_lmhead_op, "extern \"C\" __device__ void mk_lmhead_op(const void* view, const MkInstr* instr);");
+PL_SERVE(op_lmhead, "op_lmhead");
+PL_USES("pipelink_mk_vec");
+PL_PRELUDE("include/mk_abi.h");
+PL_EMIT_MAIN()

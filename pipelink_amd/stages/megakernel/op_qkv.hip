@@ -1,0 +1,30 @@
+// Package mk.qkv: qkv = Wqkv[layer] . vector; this workgroup's share of the (HQ + 2 HKV) * 64 rows.
+#include <pipelink/stage.hpp>
+#ifndef PIPELINK_EMIT
+#include "mk_device.hpp"
+
+extern "C" __device__ void mk_qkv_op(const void* view, const MkInstr* instr) {
+  const MkModel& m = mk::model(view);
+  const uint16_t* w = mk::layer_of(m, instr->layer).wqkv;
+  const float* x = mk::vec();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int first, last;
+  mk::my_rows((m.hq + 2 * m.hkv) * MK_HEAD_DIM, first, last);
+  for (int r = first + wave; r < last; r += 4) {
+    const float v = mk::row_dot(w + (int64_t)r * m.d, x, m.d, lane);
+    if (lane == 0) m.qkv[r] = v;
+  }
+}
+#else
+#include "include/mk_abi.h"
+#endif
+
+PL_STAGE("mk.qkv", "0.1.0");
+PL_NO_PARAMS();
+PL_TOPOLOGY(true, "static");
+PL_VARIANT(0, {});
+PL_EXPORT(op_qkv, mk_qkv_op, "extern \"C\" __device__ void mk_qkv_op(const void* view, const MkInstr* instr);");
+PL_SERVE(op_qkv, "op_qkv");
+PL_USES("pipelink_mk_vec");
+PL_PRELUDE("include/mk_abi.h");
+PL_EMIT_MAIN()

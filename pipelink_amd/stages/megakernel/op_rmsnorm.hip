@@ -1,0 +1,39 @@
+// Package mk.rmsnorm: vector = x * rsqrt(mean(x^2) + eps) * weight into the workgroup's LDS vector.  Every
+// workgroup normalises the whole residual for itself (D floats): cheaper than a grid barrier.
+#include <pipelink/stage.hpp>
+#ifndef PIPELINK_EMIT
+#include "mk_device.hpp"
+
+extern "C" __device__ void mk_rmsnorm_op(const void* view, const MkInstr* instr) {
+  const MkModel& m = mk::model(view);
+  const uint16_t* weight = instr->opcode == MK_OP_RMSNORM_FINAL ? mk::final_norm(m)
+                           : instr->opcode == MK_OP_RMSNORM_FFN ? mk::layer_of(m, instr->layer).ffn_norm
+                                                                : mk::layer_of(m, instr->layer).attn_norm;
+  float* out = mk::vec();
+  float* scratch = out + m.d;  // 4 floats behind the vector (the vector region holds at least D + 64 floats)
+  const int tid = threadIdx.x;
+  float ss = 0.0f;
+  for (int i = tid; i < m.d; i += MK_THREADS) {
+    const float v = m.x[i];
+    out[i] = v;
+    ss += v * v;
+  }
+  ss = mk::wave_sum(ss);
+  if ((tid & 63) == 0) scratch[tid >> 6] = ss;
+  __syncthreads();
+  const float inv = __builtin_amdgcn_rsqf((scratch[0] + scratch[1] + scratch[2] + scratch[3]) / (float)m.d + m.eps);
+  for (int i = tid; i < m.d; i += MK_THREADS) out[i] = out[i] * inv * mk::bf16_to_f32(weight[i]);
+}
+#else
+#include "include/mk_abi.h"
+#endif
+
+PL_STAGE("mk.rmsnorm", "0.1.0");
+PL_NO_PARAMS();
+PL_TOPOLOGY(true, "static");
+PL_VARIANT(0, {});
+PL_EXPORT(op_rmsnorm, mk_rmsnorm_op, "extern \"C\" __device__ void mk_rmsnorm_op(const void* view, const MkInstr* instr);");
+PL_SERVE(op_rmsnorm, "op_rmsnorm");
+PL_USES("pipelink_mk_vec");
+PL_PRELUDE("include/mk_abi.h");
+PL_EMIT_MAIN()

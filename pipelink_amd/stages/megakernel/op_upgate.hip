@@ -1,0 +1,31 @@
+// Package mk.upgate: h = silu(Wgate . vector) * (Wup . vector) for this workgroup's share of the DFF rows.
+#include <pipelink/stage.hpp>
+#ifndef PIPELINK_EMIT
+#include "mk_device.hpp"
+
+extern "C" __device__ void mk_upgate_op(const void* view, const MkInstr* instr) {
+  const MkModel& m = mk::model(view);
+  const mk::Layer l = mk::layer_of(m, instr->layer);
+  const float* x = mk::vec();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int first, last;
+  mk::my_rows(m.dff, first, last);
+  for (int r = first + wave; r < last; r += 4) {
+    float g, u;
+    mk::row_dot2(l.wgate + (int64_t)r * m.d, l.wup + (int64_t)r * m.d, x, m.d, lane, g, u);
+    if (lane == 0) m.h[r] = g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f)) * u;
+  }
+}
+#else
+#include "include/mk_abi.h"
+#endif
+
+PL_STAGE("mk.upgate", "0.1.0");
+PL_NO_PARAMS();
+PL_TOPOLOGY(true, "static");
+PL_VARIANT(0, {});
+PL_EXPORT(op_upgate, mk_upgate_op, "extern \"C\" __device__ void mk_upgate_op(const void* view, const MkInstr* instr);");
+PL_SERVE(op_upgate, "op_upgate");
+PL_USES("pipelink_mk_vec");
+PL_PRELUDE("include/mk_abi.h");
+PL_EMIT_MAIN()

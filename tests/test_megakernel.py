@@ -1,0 +1,154 @@
+"""Decode megakernel: an interpreter package and eight op packages linked into one persistent kernel that runs
+a whole decoding step; swapping only the attention package and relinking.
+
+CPU part: the oracle's pins, the instruction stream, what the two links record.  GPU part (marked gpu): a small
+model against the oracle (logits, residual stream, the appended cache rows), linked vs one-unit byte-identical,
+the swapped attention within tolerance of the first; then the stated model (16 layers, d 2048, 32 / 8 heads of 64,
+d_ff 8192, vocabulary 128256, 4096 cached positions) against the oracle, with its time per token."""
+import json
+import shutil
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import llama_decode as ld
+from pipelink_amd.stages.megakernel import build as mk_build
+from pipelink_amd.stages.megakernel import params as mkp
+
+ROOT = Path(__file__).resolve().parents[1]
+needs_rocm = pytest.mark.skipif(shutil.which("hipcc") is None and not Path("/opt/rocm/bin/hipcc").exists(),
+                                reason="needs the ROCm toolchain")
+SMALL = dict(layers=2, d=512, hq=8, hkv=2, dff=1024, vocab=1000, pos=37)
+
+
+def test_oracle_pieces_against_library_routines_and_invariants():
+    g = torch.Generator().manual_seed(0)
+    x, w = torch.randn(512, generator=g), (1 + 0.02 * torch.randn(512, generator=g)).to(torch.bfloat16)
+    assert torch.allclose(ld.rms_norm(x, w, 1e-5), torch.nn.functional.rms_norm(x, (512,), w.float(), 1e-5), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(ld.silu(x), torch.nn.functional.silu(x), rtol=1e-5, atol=1e-6)
+    q, k = torch.randn(64, generator=g), torch.randn(64, generator=g)
+    assert torch.allclose(ld.rope(q, 123).norm(), q.norm(), rtol=1e-5)                    # a rotation
+    assert torch.allclose(ld.rope(q, 0), q)
+    a = ld.rope(q, 100) @ ld.rope(k, 90)
+    b = ld.rope(q, 40) @ ld.rope(k, 30)
+    assert torch.allclose(a, b, rtol=1e-4, atol=1e-4)                                      # depends on the distance only
+    assert np.allclose(mkp.rope_table(123)[0], np.cos(123 * 500000.0 ** (-np.arange(0, 64, 2) / 64)), atol=1e-6)
+
+
+def test_oracle_attention_against_the_library():
+    cfg = dict(SMALL, smax=64)
+    weights, cache, x = ld.make_model(**cfg, seed=1)
+    logits, x2 = ld.decode_step(weights, cache.clone(), x, **SMALL)
+    assert torch.isfinite(logits).all() and logits.shape == (1000,) and not torch.equal(x2, x)
+    # one head of layer 0 by hand through scaled_dot_product_attention
+    w = ld.layer_views(weights, 0, 512, 8, 2, 1024)
+    qkv = w["wqkv"].float() @ ld.rms_norm(x, w["attn_norm"], 1e-5)
+    q = ld.rope(qkv[:512].view(8, 64), 37)
+    c = cache.clone()
+    ld.decode_step(weights, c, x, **SMALL)
+    keys, vals = c[0, 0, :38, 1].float(), c[0, 1, :38, 1].float()     # KV head 1 serves query heads 4..7
+    lib = torch.nn.functional.scaled_dot_product_attention(q[5][None, None], keys[None], vals[None])[0, 0]
+    mine = torch.softmax((keys @ q[5]) / 8.0, 0) @ vals
+    assert torch.allclose(lib, mine, rtol=1e-5, atol=1e-6)
+    assert weights.numel() == 2 * mkp.layer_elems(512, 8, 2, 1024) + 512 + 1000 * 512
+
+
+def test_program_is_the_whole_step():
+    p = mkp.program(16)
+    assert p.shape == (16 * 7 + 2, 4) and p.dtype == np.int32
+    assert p[:, 2].sum() == 16 * 5                       # five grid barriers per layer
+    assert list(p[:7, 0]) == [1, 2, 3, 4, 5, 6, 7] and list(p[-2:, 0]) == [8, 9] and p[-1, 2] == 0
+    assert len(mkp.params_blob({k: 0 for k in ("weights", "kv_cache", "x", "qkv", "attn_partial", "h", "logits", "rope", "program", "sync")},
+                               num_instr=3, layers=1, d=512, hq=8, hkv=2, dff=1024, vocab=10, pos=1, smax=4, chunks=1)) == 128
+
+
+@pytest.fixture(scope="module")
+def example(tmp_path_factory):
+    out = tmp_path_factory.mktemp("megakernel")
+    return out, mk_build.build(out=out, one_unit=False)
+
+
+@needs_rocm
+def test_links_nine_packages_and_swaps_only_the_attention(example):
+    out, res = example
+    link, swap = res["link"], res["swap"]
+    assert link["params"]["entries"] == [{"stage_id": "mk.interp", "offset": 0, "bytes": 128, "align": 8}]
+    assert link["threads"] == 256 and link["dyn_smem_bytes"] == 32768
+    assert {e["channel"] for e in link["protocol_expansions"]} == {"op_rmsnorm", "op_qkv", "op_attn", "op_oproj", "op_upgate", "op_down",
+                                                                   "op_lmhead", "rope_apply"}
+    assert link["observed"]["calls"] == 0 and swap["observed"]["calls"] == 0
+    same = set(link["input_hashes"]) & set(swap["input_hashes"])
+    assert same == {"mk.interp", "mk.rmsnorm", "mk.qkv", "mk.rope", "mk.oproj", "mk.upgate", "mk.down", "mk.lmhead"}
+    assert all(link["input_hashes"][s] == swap["input_hashes"][s] for s in same)            # eight packages untouched
+    assert "mk.attn" in link["input_hashes"] and "mk.attn.wide" in swap["input_hashes"]
+
+
+# ---- GPU ---------------------------------------------------------------------------------------------------
+
+def _bits(t: torch.Tensor) -> np.ndarray:
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _run(paths_key, cfg, weights, cache, x, workgroups, image_key=None, time_launches=0):
+    from pipelink_amd.host.megakernel import open_session
+
+    paths = mk_build.images()
+    sess = open_session(paths[paths_key], _bits(weights), _bits(cache), x.numpy(), workgroups=workgroups, **cfg,
+                        image=paths[image_key] if image_key else None)
+    try:
+        sess.launch()
+        sess.synchronize()
+        out = {n: sess.read(n) for n in ("logits", "x", "kv_cache", "sync")}
+        if time_launches:
+            out["ms"] = sess.time(time_launches)
+            out["sync_after_timing"] = sess.read("sync")
+        return out
+    finally:
+        sess.close()
+
+
+def _rel(a, b):
+    return float(np.linalg.norm(a - b) / np.linalg.norm(b))
+
+
+@pytest.mark.gpu
+def test_small_model_matches_the_oracle_linked_one_unit_and_swapped():
+    cfg = dict(SMALL)
+    weights, cache, x = ld.make_model(**cfg, smax=64, seed=2)
+    ref_cache = cache.clone()
+    want_logits, want_x = ld.decode_step(weights, ref_cache, x, **cfg)
+    got = _run("link_json", cfg, weights, cache, x, workgroups=32)
+    assert list(got["sync"][:3]) == [0, 0, 0], "a grid barrier gave up or the counters were not put back"
+    assert _rel(got["x"], want_x.numpy()) <= 2e-3 and _rel(got["logits"], want_logits.numpy()) <= 2e-3
+    assert int(np.argmax(got["logits"])) == int(torch.argmax(want_logits))
+    new_rows = got["kv_cache"][:, :, 37]                                      # the appended key and value of both layers
+    ref_rows = _bits(ref_cache)[:, :, 37]
+    assert (new_rows != ref_rows).mean() < 0.02                               # bf16 roundings of fp32 sums in another order
+    near = torch.from_numpy(new_rows.view(np.int16).copy()).view(torch.bfloat16).float().numpy()
+    assert _rel(near, ref_cache[:, :, 37].float().numpy()) <= 1e-2
+    assert np.array_equal(got["kv_cache"][:, :, :37], _bits(cache)[:, :, :37])  # the rest of the cache untouched
+    control = _run("link_json", cfg, weights, cache, x, workgroups=32, image_key="one_unit")
+    assert all(np.array_equal(control[n], got[n]) for n in ("logits", "x", "kv_cache")), "linked and one-unit images differ"
+    swapped = _run("swap_link_json", cfg, weights, cache, x, workgroups=32)
+    assert list(swapped["sync"][:3]) == [0, 0, 0]
+    assert _rel(swapped["logits"], got["logits"]) <= 1e-4 and _rel(swapped["logits"], want_logits.numpy()) <= 2e-3
+
+
+@pytest.mark.gpu
+def test_stated_model_against_the_oracle_and_its_time_per_token():
+    cfg = dict(layers=16, d=2048, hq=32, hkv=8, dff=8192, vocab=128256, pos=4096)
+    weights, cache, x = ld.make_model(**cfg, smax=4104, seed=0)
+    print(f"weights {weights.numel() * 2 / 1e9:.2f} GB, cache {cache.numel() * 2 / 1e6:.0f} MB", flush=True)
+    want_logits, want_x = ld.decode_step(weights, cache.clone(), x, **cfg)
+    got = _run("link_json", cfg, weights, cache, x, workgroups=256, time_launches=20)
+    assert list(got["sync"][:3]) == [0, 0, 0] and list(got["sync_after_timing"][:3]) == [0, 0, 0]
+    assert _rel(got["x"], want_x.numpy()) <= 5e-3 and _rel(got["logits"], want_logits.numpy()) <= 5e-3
+    assert int(np.argmax(got["logits"])) == int(torch.argmax(want_logits))
+    bytes_per_token = weights.numel() * 2 + cache[:, :, :4096].numel() * 2
+    print(f"decode step: {got['ms']:.3f} ms per token, {bytes_per_token / got['ms'] / 1e9:.2f} TB/s of {bytes_per_token / 1e9:.2f} GB "
+          f"(weights + cache read once), {bytes_per_token / got['ms'] / 1e9 / 8 * 100:.1f} % of 8 TB/s", flush=True)
+    swapped = _run("swap_link_json", cfg, weights, cache, x, workgroups=256, time_launches=20)
+    assert _rel(swapped["logits"], got["logits"]) <= 1e-4
+    print(f"with mk.attn.wide relinked: {swapped['ms']:.3f} ms per token", flush=True)
