@@ -21,13 +21,17 @@ def open_session(link_json: str | Path, weights: np.ndarray, kv_cache: np.ndarra
         raise ValueError("weights do not have the packed size for these dimensions")
     if d % 512 or dff % 512 or (hq * mk.HEAD_DIM) % 512 or hq % hkv or workgroups % hq or pos >= smax or d + 64 > 8192 or dff > 8192:
         raise ValueError("d, dff and hq*64 must be multiples of 512 (dff <= 8192), hq a multiple of hkv, workgroups a multiple of hq, pos < smax")
+    if dff % (4 * workgroups):
+        raise ValueError("dff must be a multiple of 4 * workgroups")
     chunks = workgroups // hq
+    if hq * mk.HEAD_DIM + 3 * workgroups > 8192 + 256:
+        raise ValueError("the attention output and the chunk weights do not fit the workgroup's LDS vector")
     if (pos + 1 + chunks - 1) // chunks > 8192 - 512:
         raise ValueError("a context chunk does not fit the workgroup's LDS vector: use more workgroups")
     prog = mk.program(layers)
     buffers = {"weights": weights, "kv_cache": kv_cache, "x": x.astype(np.float32), "rope": mk.rope_table(pos), "program": prog,
-               "qkv": (((hq + 2 * hkv) * mk.HEAD_DIM,), np.float32), "attn_partial": ((hq * chunks * (mk.HEAD_DIM + 2),), np.float32),
-               "h": ((dff,), np.float32), "logits": ((vocab,), np.float32), "sync": ((4,), np.uint32)}
+               "qkv": (((hq + 2 * hkv) * mk.HEAD_DIM,), np.float32), "attn_partial": ((hq * chunks * mk.PARTIAL_STRIDE,), np.float32),
+               "h": ((dff,), np.float32), "logits": ((vocab,), np.float32), "sync": ((512,), np.uint32)}
     blob = lambda addr: {"mk.interp": mk.params_blob(addr, num_instr=len(prog), layers=layers, d=d, hq=hq, hkv=hkv, dff=dff,
                                                      vocab=vocab, pos=pos, smax=smax, chunks=chunks)}
     return open_hostless(link_json, buffers=buffers, params=blob, grid=(workgroups,), backend=backend, image=image)

@@ -19,6 +19,9 @@
 
 #define MK_THREADS 256
 #define MK_HEAD_DIM 64
+// floats per (head, context chunk) of the attention partials: 64 unnormalised outputs, the chunk's maximum (log2
+// units), its sum of exponentials, two floats of padding (rows stay 16-byte aligned)
+#define MK_PARTIAL_STRIDE (MK_HEAD_DIM + 4)
 
 enum {
   MK_OP_RMSNORM_ATTN = 1, /* x * rsqrt(mean x^2 + eps) * attn_norm[layer]  -> LDS vector */
@@ -49,7 +52,8 @@ typedef struct MkModel {
   const float* rope;       /* [2][32]: cos, sin of pos * theta^(-2 i / 64) */
   const MkInstr* program;
   uint32_t* sync;          /* [0] grid barrier counter (zero at launch; the kernel leaves it zero), [1] status (non-zero: a
-                              wait gave up), [2] count of workgroups that have finished (zero at launch, left zero) */
+                              wait gave up), [2] count of workgroups that have finished, [32 * (1 + xcd)] arrivals of
+                              one XCD's workgroups; 512 words, all zero at launch and left zero */
   int32_t num_instr, layers, d, hq, hkv, dff, vocab, pos, smax, chunks;
   float eps, attn_scale_log2e;
 } MkModel;

@@ -3,8 +3,7 @@
 // One workgroup per CU, all resident at once.  Every workgroup walks the same instruction stream
 // (MkModel.program); an instruction names an op, the op's package does this workgroup's share of it.
 // Where an instruction asks for it, the workgroups meet at a grid barrier: a counter in global memory
-// that only grows (barrier n is passed when it reaches n * workgroups), arrived at with an agent-scope
-// release and left with an acquire, so that what one workgroup wrote (on any XCD) is what the others read.
+// that only grows, so that what one workgroup wrote (on any XCD) before it is what the others read after it.
 // The wait is a bounded poll: a workgroup that gives up raises the status word and goes on, it never
 // spins for ever.
 #include <pipelink/stage.hpp>
@@ -22,24 +21,52 @@ extern "C" __device__ void pipelink_call_op_lmhead(const void* view, const MkIns
 namespace mk_interp {
 constexpr uint32_t SPIN_LIMIT = 1u << 22;
 
+// Arrival and release are both in two levels.  An atomic or a load that every XCD must agree on is performed at
+// the memory side, one after the other: 256 of them on one word cost more than the work between two barriers.
+// So a workgroup first arrives on its XCD's own counter (workgroups are dealt to the 8 XCDs round-robin,
+// blockIdx % 8; an access at workgroup scope is served by that XCD's L2), and only the last arrival of an XCD
+// goes on to the grid's counter.  One workgroup per XCD polls the grid's counter and then passes the word on to
+// its XCD in a generation number the others poll in their L2.  No cache is written back or invalidated here: what
+// workgroups hand each other across a barrier is stored and loaded at device scope (mk::shared_store / shared_load),
+// and every wave has waited for its stores (the __syncthreads) before its workgroup is counted.
+constexpr int NUM_XCD = 8;
+constexpr int XCD_COUNTER = 32;      // sync[32 * (1 + xcd)]: arrivals; [32 * (1 + xcd) + 1]: generation; one 128-byte line per XCD
+__device__ __forceinline__ bool poll(uint32_t* word, uint32_t target, bool local, const MkModel& m) {
+  for (uint32_t spin = 0; spin < SPIN_LIMIT; ++spin) {
+    // local: an atomic add of 0 written out as such -- atomics are performed in the L2, whereas a plain
+    // workgroup-scope load (which the compiler makes of an idempotent read-modify-write) could be served by
+    // this CU's L1 for ever
+    uint32_t seen;
+    if (local) {
+      const uint32_t zero = 0;
+      asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)" : "=&v"(seen) : "v"(word), "v"(zero) : "memory");
+    } else {
+      seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if ((int32_t)(seen - target) >= 0) return true;
+    __builtin_amdgcn_s_sleep(1);
+  }
+  __hip_atomic_fetch_or(m.sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return false;
+}
 __device__ __forceinline__ void grid_barrier(const MkModel& m, uint32_t& passed) {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // this wave's stores, visible device-wide
-  __syncthreads();
+  __syncthreads();  // every wave's stores have been issued and acknowledged by the L2
   ++passed;
   if (threadIdx.x == 0) {
-    const uint32_t target = passed * gridDim.x;
-    __hip_atomic_fetch_add(m.sync, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-    uint32_t spin = 0;
-    while ((int32_t)(__hip_atomic_load(m.sync, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
-      if (++spin >= SPIN_LIMIT) {
-        __hip_atomic_fetch_or(m.sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        break;
-      }
-      __builtin_amdgcn_s_sleep(2);
+    const uint32_t xcd = blockIdx.x % NUM_XCD;
+    const uint32_t members = (gridDim.x - xcd + NUM_XCD - 1) / NUM_XCD, groups = min((uint32_t)NUM_XCD, gridDim.x);
+    uint32_t* mine = m.sync + XCD_COUNTER * (1 + xcd);
+    const uint32_t before = __hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (before + 1 == passed * members)
+      __hip_atomic_fetch_add(m.sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (blockIdx.x < NUM_XCD) {  // this XCD's first workgroup listens for the grid
+      poll(m.sync, passed * groups, false, m);
+      __hip_atomic_exchange(mine + 1, passed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    } else {
+      poll(mine + 1, passed, true, m);
     }
   }
   __syncthreads();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // nothing cached from before the barrier is read after it
 }
 }  // namespace mk_interp
 
@@ -71,6 +98,10 @@ extern "C" __device__ void mk_interp_role_worker(const void* params, unsigned va
     const uint32_t before = __hip_atomic_fetch_add(m.sync + 2, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
     if (before == gridDim.x - 1) {
       __hip_atomic_store(m.sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int x = 0; x < mk_interp::NUM_XCD; ++x) {
+        __hip_atomic_store(m.sync + mk_interp::XCD_COUNTER * (1 + x), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(m.sync + mk_interp::XCD_COUNTER * (1 + x) + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
       __hip_atomic_store(m.sync + 2, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
@@ -93,8 +124,9 @@ MK_CALL(upgate);
 MK_CALL(down);
 MK_CALL(lmhead);
 // the workgroup's activation vector: the normalised residual (D floats), the attention output (HQ * 64) or
-// the FFN intermediate (DFF floats), whichever the running op needs; 32 KB holds DFF = 8192
-PL_CLAIM("pipelink_mk_vec", "smem", 32768, 1024, "kernel");
+// the FFN intermediate (DFF floats), whichever the running op needs; 32 KB holds DFF = 8192, and 1 KB behind it is
+// the ops' reduction scratch
+PL_CLAIM("pipelink_mk_vec", "smem", 33792, 1024, "kernel");
 PL_USES("pipelink_mk_vec");
 PL_PRELUDE("include/mk_abi.h");
 PL_EMIT_MAIN()

@@ -71,26 +71,54 @@ extern "C" __device__ void mk_attn_op(const void* view, const MkInstr* instr) {
   local_sum = mk::wave_sum(local_sum);
   if (lane == 0) red[4 + wave] = local_sum;
   __syncthreads();
-  // ---- unnormalised output: lane = d, a wave takes every fourth position ------------------------------------
-  float o = 0.0f;
-  for (int p = p0 + wave; p < p1; p += 4) {
-    const float v = p < m.pos ? mk::bf16_to_f32(vc[p * pos_stride + lane]) : mk_attn::bf16_round(vnew[lane]);
-    o += score[p - p0] * v;
+  // ---- unnormalised output: 16 lanes take one position (four d each, one 8-byte load), a wave four positions per
+  // load instruction and sixteen such loads in flight ------------------------------------------------------
+  {
+    const int g = lane >> 4, dq = lane & 15;
+    const int cached_end = min(p1, m.pos), last_cached = max(m.pos - 1, 0);
+    float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int pb = p0 + 4 * wave + g; pb < cached_end; pb += 16 * 16) {
+      uint2 v[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) v[j] = *reinterpret_cast<const uint2*>(vc + min(pb + 16 * j, last_cached) * pos_stride + 4 * dq);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int p = pb + 16 * j;
+        const float s = p < cached_end ? score[p - p0] : 0.0f;
+        o[0] += s * mk::bf16_to_f32(v[j].x & 0xFFFFu);
+        o[1] += s * __uint_as_float(v[j].x & 0xFFFF0000u);
+        o[2] += s * mk::bf16_to_f32(v[j].y & 0xFFFFu);
+        o[3] += s * __uint_as_float(v[j].y & 0xFFFF0000u);
+      }
+    }
+    if (p0 <= m.pos && m.pos < p1 && wave == 0 && g == 0) {  // the step's own token, as the cache will hold it
+      const float s = score[m.pos - p0];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] += s * mk_attn::bf16_round(mk::shared_load(vnew + 4 * dq + e));
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      o[e] += __shfl_xor(o[e], 16);
+      o[e] += __shfl_xor(o[e], 32);
+    }
+    if (g == 0) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) part[wave * 64 + 4 * dq + e] = o[e];
+    }
   }
-  part[wave * 64 + lane] = o;
   __syncthreads();
-  float* out = m.attn_partial + ((int64_t)head * m.chunks + chunk) * (MK_HEAD_DIM + 2);
-  if (tid < 64) out[tid] = part[tid] + part[64 + tid] + part[128 + tid] + part[192 + tid];
+  float* out = m.attn_partial + ((int64_t)head * m.chunks + chunk) * MK_PARTIAL_STRIDE;
+  if (tid < 64) mk::shared_store(out + tid, part[tid] + part[64 + tid] + part[128 + tid] + part[192 + tid]);
   if (tid == 64) {
-    out[MK_HEAD_DIM] = cmax;
-    out[MK_HEAD_DIM + 1] = red[4] + red[5] + red[6] + red[7];
+    mk::shared_store(out + MK_HEAD_DIM, cmax);
+    mk::shared_store(out + MK_HEAD_DIM + 1, red[4] + red[5] + red[6] + red[7]);
   }
   // ---- append the step's key and value (one workgroup per KV head does it) ----------------------------------
   if (head % (m.hq / m.hkv) == 0 && p0 <= m.pos && m.pos < p1 && tid < 64) {
     uint16_t* kdst = m.kv_cache + (((int64_t)instr->layer * 2 + 0) * m.smax + m.pos) * pos_stride + kvh * MK_HEAD_DIM;
     uint16_t* vdst = m.kv_cache + (((int64_t)instr->layer * 2 + 1) * m.smax + m.pos) * pos_stride + kvh * MK_HEAD_DIM;
     kdst[tid] = (uint16_t)(__float_as_uint(knew[tid]) >> 16);
-    vdst[tid] = (uint16_t)(__float_as_uint(mk_attn::bf16_round(vnew[tid])) >> 16);
+    vdst[tid] = (uint16_t)(__float_as_uint(mk_attn::bf16_round(mk::shared_load(vnew + tid))) >> 16);
   }
 }
 #else

@@ -41,11 +41,30 @@ extern "C" __device__ void mk_attn_wide_op(const void* view, const MkInstr* inst
   __syncthreads();
   // ---- scores (log2 units) and the chunk's maximum ---------------------------------------------------------
   float local_max = -1.0e30f;
-  for (int p = p0 + wave; p < p1; p += 4) {
-    const float kv = p < m.pos ? mk::bf16_to_f32(kc[p * pos_stride + lane]) : knew[lane];
-    const float sc = mk::wave_sum(kv * q[lane]) * m.attn_scale_log2e;
-    if (lane == 0) score[p - p0] = sc;
-    local_max = fmaxf(local_max, sc);
+  {
+    const float ql = q[lane];
+    int p = p0 + wave;
+    for (; p + 28 < p1 && p + 28 < m.pos; p += 32) {
+      float kv[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) kv[j] = mk::bf16_to_f32(kc[(p + 4 * j) * pos_stride + lane]) * ql;
+#pragma unroll
+      for (int sh = 32; sh >= 1; sh >>= 1)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) kv[j] += __shfl_xor(kv[j], sh);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float sc = kv[j] * m.attn_scale_log2e;
+        if (lane == 0) score[p + 4 * j - p0] = sc;
+        local_max = fmaxf(local_max, sc);
+      }
+    }
+    for (; p < p1; p += 4) {
+      const float kv = p < m.pos ? mk::bf16_to_f32(kc[p * pos_stride + lane]) : knew[lane];
+      const float sc = mk::wave_sum(kv * ql) * m.attn_scale_log2e;
+      if (lane == 0) score[p - p0] = sc;
+      local_max = fmaxf(local_max, sc);
+    }
   }
   __syncthreads();
 #pragma unroll
@@ -64,24 +83,34 @@ extern "C" __device__ void mk_attn_wide_op(const void* view, const MkInstr* inst
   __syncthreads();
   // ---- unnormalised output: lane = d, a wave takes every fourth position ------------------------------------
   float o = 0.0f;
-  for (int p = p0 + wave; p < p1; p += 4) {
-    const float v = p < m.pos ? mk::bf16_to_f32(vc[p * pos_stride + lane]) : mk_attn_wide::bf16_round(vnew[lane]);
-    o += score[p - p0] * v;
+  {
+    int p = p0 + wave;
+    for (; p + 28 < p1 && p + 28 < m.pos; p += 32) {  // eight cached positions at a time: eight loads in flight
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = mk::bf16_to_f32(vc[(p + 4 * j) * pos_stride + lane]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o += score[p + 4 * j - p0] * v[j];
+    }
+    for (; p < p1; p += 4) {
+      const float v = p < m.pos ? mk::bf16_to_f32(vc[p * pos_stride + lane]) : mk_attn_wide::bf16_round(mk::shared_load(vnew + lane));
+      o += score[p - p0] * v;
+    }
   }
   part[wave * 64 + lane] = o;
   __syncthreads();
-  float* out = m.attn_partial + ((int64_t)head * m.chunks + chunk) * (MK_HEAD_DIM + 2);
-  if (tid < 64) out[tid] = part[tid] + part[64 + tid] + part[128 + tid] + part[192 + tid];
+  float* out = m.attn_partial + ((int64_t)head * m.chunks + chunk) * MK_PARTIAL_STRIDE;
+  if (tid < 64) mk::shared_store(out + tid, part[tid] + part[64 + tid] + part[128 + tid] + part[192 + tid]);
   if (tid == 64) {
-    out[MK_HEAD_DIM] = cmax;
-    out[MK_HEAD_DIM + 1] = red[4] + red[5] + red[6] + red[7];
+    mk::shared_store(out + MK_HEAD_DIM, cmax);
+    mk::shared_store(out + MK_HEAD_DIM + 1, red[4] + red[5] + red[6] + red[7]);
   }
   // ---- append the step's key and value (one workgroup per KV head does it) ----------------------------------
   if (head % (m.hq / m.hkv) == 0 && p0 <= m.pos && m.pos < p1 && tid < 64) {
     uint16_t* kdst = m.kv_cache + (((int64_t)instr->layer * 2 + 0) * m.smax + m.pos) * pos_stride + kvh * MK_HEAD_DIM;
     uint16_t* vdst = m.kv_cache + (((int64_t)instr->layer * 2 + 1) * m.smax + m.pos) * pos_stride + kvh * MK_HEAD_DIM;
     kdst[tid] = (uint16_t)(__float_as_uint(knew[tid]) >> 16);
-    vdst[tid] = (uint16_t)(__float_as_uint(mk_attn_wide::bf16_round(vnew[tid])) >> 16);
+    vdst[tid] = (uint16_t)(__float_as_uint(mk_attn_wide::bf16_round(mk::shared_load(vnew + tid))) >> 16);
   }
 }
 #else

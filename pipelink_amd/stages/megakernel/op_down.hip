@@ -7,15 +7,19 @@
 extern "C" __device__ void mk_down_op(const void* view, const MkInstr* instr) {
   const MkModel& m = mk::model(view);
   float* hv = mk::vec();
-  for (int i = threadIdx.x; i < m.dff; i += MK_THREADS) hv[i] = m.h[i];
+  for (int i = 4 * threadIdx.x; i < m.dff; i += 4 * MK_THREADS) *reinterpret_cast<mk::v4f*>(hv + i) = mk::shared_load4(m.h, i, m.dff);
   __syncthreads();
   const uint16_t* w = mk::layer_of(m, instr->layer).wdown;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float* scratch = hv + 8192;  // behind the vector
   int first, last;
   mk::my_rows(m.d, first, last);
-  for (int r = first + wave; r < last; r += 4) {
-    const float v = mk::row_dot(w + (int64_t)r * m.dff, hv, m.dff, lane);
-    if (lane == 0) m.x[r] += v;
+  for (int r = first; r < last; r += 8) {
+    const int count = min(8, last - r);
+    if (count == 8) {
+      mk::matvec_split<8>(w + (int64_t)r * m.dff, m.dff, hv, scratch, 8, [&](int i, float v) { mk::shared_store(m.x + r + i, mk::shared_load(m.x + r + i) + v); });
+    } else {
+      mk::matvec<1>(w, m.dff, hv, r, last, [&](int row, float v) { mk::shared_store(m.x + row, mk::shared_load(m.x + row) + v); });
+    }
   }
 }
 #else

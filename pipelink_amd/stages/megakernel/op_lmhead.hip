@@ -8,22 +8,9 @@ extern "C" __device__ void mk_lmhead_op(const void* view, const MkInstr* instr) 
   const MkModel& m = mk::model(view);
   const uint16_t* w = mk::lm_head(m);
   const float* x = mk::vec();
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int first, last;
   mk::my_rows(m.vocab, first, last);
-  int r = first + 2 * wave;
-  for (; r + 1 < last; r += 8) {
-    float a, b;
-    mk::row_dot2(w + (int64_t)r * m.d, w + (int64_t)(r + 1) * m.d, x, m.d, lane, a, b);
-    if (lane == 0) {
-      m.logits[r] = a;
-      m.logits[r + 1] = b;
-    }
-  }
-  if (r < last) {
-    const float a = mk::row_dot(w + (int64_t)r * m.d, x, m.d, lane);
-    if (lane == 0) m.logits[r] = a;
-  }
+  mk::matvec<4>(w, m.d, x, first, last, [&](int r, float v) { m.logits[r] = v; });
 }
 #else
 #include "include/mk_abi.h"

@@ -9,28 +9,42 @@ extern "C" __device__ void mk_oproj_op(const void* view, const MkInstr* instr) {
   const MkModel& m = mk::model(view);
   float* a = mk::vec();
   const int n = m.hq * MK_HEAD_DIM;
-  for (int idx = threadIdx.x; idx < n; idx += MK_THREADS) {
-    const int head = idx / MK_HEAD_DIM, d = idx % MK_HEAD_DIM;
-    const float* p = m.attn_partial + (int64_t)head * m.chunks * (MK_HEAD_DIM + 2);
-    float top = -1.0e30f;
-    for (int c = 0; c < m.chunks; ++c) top = fmaxf(top, p[c * (MK_HEAD_DIM + 2) + MK_HEAD_DIM]);
-    float o = 0.0f, l = 0.0f;
-    for (int c = 0; c < m.chunks; ++c) {
-      const float w = __builtin_amdgcn_exp2f(p[c * (MK_HEAD_DIM + 2) + MK_HEAD_DIM] - top);
-      o += w * p[c * (MK_HEAD_DIM + 2) + d];
-      l += w * p[c * (MK_HEAD_DIM + 2) + MK_HEAD_DIM + 1];
+  // per (head, chunk): its weight exp2(max_c - max) / sum in the softmax over the whole context, into LDS behind the vector
+  const int pairs = m.hq * m.chunks, count = pairs * MK_PARTIAL_STRIDE;
+  float* cmax = a + n;
+  float* csum = cmax + pairs;
+  float* weight = csum + pairs;
+  for (int i = threadIdx.x; i < pairs; i += MK_THREADS) {
+    const mk::v4f t = mk::shared_load4(m.attn_partial, i * MK_PARTIAL_STRIDE + MK_HEAD_DIM, count);
+    cmax[i] = t.x;
+    csum[i] = t.y;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < pairs; i += MK_THREADS) {
+    const int first_of_head = i / m.chunks * m.chunks;
+    float top = -1.0e30f, l = 0.0f;
+    for (int c = 0; c < m.chunks; ++c) top = fmaxf(top, cmax[first_of_head + c]);
+    for (int c = 0; c < m.chunks; ++c) l += __builtin_amdgcn_exp2f(cmax[first_of_head + c] - top) * csum[first_of_head + c];
+    weight[i] = __builtin_amdgcn_exp2f(cmax[i] - top) / l;
+  }
+  __syncthreads();
+  for (int item = threadIdx.x; item < n / 4; item += MK_THREADS) {  // four outputs of one head per thread
+    const int head = item / (MK_HEAD_DIM / 4), d = 4 * (item % (MK_HEAD_DIM / 4));
+    mk::v4f o = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int c = 0; c < m.chunks; c += 4) {  // four chunks' loads in flight; a chunk past the last reads past the buffer: zeros
+      mk::v4f part[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) part[j] = mk::shared_load4(m.attn_partial, c + j < m.chunks ? (head * m.chunks + c + j) * MK_PARTIAL_STRIDE + d : count, count);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o += (c + j < m.chunks ? weight[head * m.chunks + c + j] : 0.0f) * part[j];
     }
-    a[idx] = o / l;
+    *reinterpret_cast<mk::v4f*>(a + 4 * item) = o;
   }
   __syncthreads();
   const uint16_t* w = mk::layer_of(m, instr->layer).wo;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int first, last;
   mk::my_rows(m.d, first, last);
-  for (int r = first + wave; r < last; r += 4) {
-    const float v = mk::row_dot(w + (int64_t)r * n, a, n, lane);
-    if (lane == 0) m.x[r] += v;
-  }
+  mk::matvec<2>(w, n, a, first, last, [&](int r, float v) { mk::shared_store(m.x + r, mk::shared_load(m.x + r) + v); });
 }
 #else
 #include "include/mk_abi.h"

@@ -7,13 +7,9 @@ extern "C" __device__ void mk_qkv_op(const void* view, const MkInstr* instr) {
   const MkModel& m = mk::model(view);
   const uint16_t* w = mk::layer_of(m, instr->layer).wqkv;
   const float* x = mk::vec();
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int first, last;
   mk::my_rows((m.hq + 2 * m.hkv) * MK_HEAD_DIM, first, last);
-  for (int r = first + wave; r < last; r += 4) {
-    const float v = mk::row_dot(w + (int64_t)r * m.d, x, m.d, lane);
-    if (lane == 0) m.qkv[r] = v;
-  }
+  mk::matvec<3>(w, m.d, x, first, last, [&](int r, float v) { mk::shared_store(m.qkv + r, v); });
 }
 #else
 #include "include/mk_abi.h"

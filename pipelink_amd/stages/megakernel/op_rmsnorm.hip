@@ -13,10 +13,10 @@ extern "C" __device__ void mk_rmsnorm_op(const void* view, const MkInstr* instr)
   float* scratch = out + m.d;  // 4 floats behind the vector (the vector region holds at least D + 64 floats)
   const int tid = threadIdx.x;
   float ss = 0.0f;
-  for (int i = tid; i < m.d; i += MK_THREADS) {
-    const float v = m.x[i];
-    out[i] = v;
-    ss += v * v;
+  for (int i = 4 * tid; i < m.d; i += 4 * MK_THREADS) {  // D is a multiple of 512
+    const mk::v4f v = mk::shared_load4(m.x, i, m.d);
+    *reinterpret_cast<mk::v4f*>(out + i) = v;
+    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
   }
   ss = mk::wave_sum(ss);
   if ((tid & 63) == 0) scratch[tid >> 6] = ss;

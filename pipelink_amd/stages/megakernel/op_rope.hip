@@ -4,12 +4,13 @@
 #ifndef PIPELINK_EMIT
 #include "mk_device.hpp"
 
-// out[i] for lane-held element i of head vector `v` (64 floats in global memory)
+// out[i] for lane-held element i of head vector `v` (64 floats of the qkv buffer)
 extern "C" __device__ float mk_rope_apply(const void* view, const float* v, int i) {
   const MkModel& m = mk::model(view);
   const int j = i & 31;
   const float c = m.rope[j], s = m.rope[32 + j];
-  return i < 32 ? v[i] * c - v[i + 32] * s : v[i] * c + v[i - 32] * s;
+  const float a = mk::shared_load(v + i), b = mk::shared_load(v + (i < 32 ? i + 32 : i - 32));
+  return i < 32 ? a * c - b * s : a * c + b * s;
 }
 #else
 #include "include/mk_abi.h"

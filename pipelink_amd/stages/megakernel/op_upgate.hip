@@ -10,10 +10,16 @@ extern "C" __device__ void mk_upgate_op(const void* view, const MkInstr* instr) 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int first, last;
   mk::my_rows(m.dff, first, last);
-  for (int r = first + wave; r < last; r += 4) {
-    float g, u;
-    mk::row_dot2(l.wgate + (int64_t)r * m.d, l.wup + (int64_t)r * m.d, x, m.d, lane, g, u);
-    if (lane == 0) m.h[r] = g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-g * 1.4426950408889634f)) * u;
+  constexpr int R = 4;
+  for (int r = first + R * wave; r < last; r += 4 * R) {  // DFF / workgroups is a multiple of 4 (the host checks)
+    float g[R], u[R];
+    mk::rows_dot<R>(l.wgate + (int64_t)r * m.d, m.d, x, m.d, lane, g);
+    mk::rows_dot<R>(l.wup + (int64_t)r * m.d, m.d, x, m.d, lane, u);
+    if (lane == 0) {
+#pragma unroll
+      for (int i = 0; i < R; ++i)
+        if (r + i < last) mk::shared_store(m.h + r + i, g[i] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-g[i] * 1.4426950408889634f)) * u[i]);
+    }
   }
 }
 #else

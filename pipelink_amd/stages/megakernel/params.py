@@ -6,6 +6,7 @@ import numpy as np
 
 OP_RMSNORM_ATTN, OP_QKV, OP_ATTN, OP_OPROJ, OP_RMSNORM_FFN, OP_UPGATE, OP_DOWN, OP_RMSNORM_FINAL, OP_LMHEAD = range(1, 10)
 HEAD_DIM = 64
+PARTIAL_STRIDE = HEAD_DIM + 4  # MK_PARTIAL_STRIDE
 
 
 def program(layers: int) -> np.ndarray:

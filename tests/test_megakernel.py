@@ -75,7 +75,7 @@ def test_links_nine_packages_and_swaps_only_the_attention(example):
     out, res = example
     link, swap = res["link"], res["swap"]
     assert link["params"]["entries"] == [{"stage_id": "mk.interp", "offset": 0, "bytes": 128, "align": 8}]
-    assert link["threads"] == 256 and link["dyn_smem_bytes"] == 32768
+    assert link["threads"] == 256 and link["dyn_smem_bytes"] == 33792
     assert {e["channel"] for e in link["protocol_expansions"]} == {"op_rmsnorm", "op_qkv", "op_attn", "op_oproj", "op_upgate", "op_down",
                                                                    "op_lmhead", "rope_apply"}
     assert link["observed"]["calls"] == 0 and swap["observed"]["calls"] == 0
