@@ -26,7 +26,7 @@ def open_session(link_json: str | Path, weights: np.ndarray, kv_cache: np.ndarra
     chunks = workgroups // hq
     if hq * mk.HEAD_DIM + 3 * workgroups > 8192 + 256:
         raise ValueError("the attention output and the chunk weights do not fit the workgroup's LDS vector")
-    if (pos + 1 + chunks - 1) // chunks > 8192 - 512:
+    if (pos + chunks - 1) // chunks + 1 > 8192 + 256 - 1280:  # the scores sit 1280 floats into the vector
         raise ValueError("a context chunk does not fit the workgroup's LDS vector: use more workgroups")
     prog = mk.program(layers)
     buffers = {"weights": weights, "kv_cache": kv_cache, "x": x.astype(np.float32), "rope": mk.rope_table(pos), "program": prog,

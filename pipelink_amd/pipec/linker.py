@@ -108,12 +108,18 @@ def _to_bitcode(source: Path, out: Path, arch: str, flags: list[str], include_di
 
 def _finalise(bitcode: Path, hsaco: Path, arch: str) -> None:
     """Internalise everything but the kernel, run the -O3 pipeline once over the merged module
-    (clang does not re-optimise IR input on its own), then emit the code object."""
+    (clang does not re-optimise IR input on its own), then emit the code object.  Where the
+    pipeline's own inliner leaves a call behind (a very large role or export), the module is
+    finalised again with every function marked always-inline: a linked kernel has no calls."""
     optimised = bitcode.with_suffix(".opt.bc")
-    _run([LLVM_BIN / "opt", "-passes=internalize,globaldce,default<O3>", f"-internalize-public-api-list={KERNEL_SYMBOL}",
-          bitcode, "-o", optimised], "link.optimise")
-    _run([LLVM_BIN / "clang", "-x", "ir", "-target", "amdgcn-amd-amdhsa", f"-mcpu={arch}", "-O3", "-nogpulib",
-          optimised, "-o", hsaco], "link.codegen")
+    for forced in ([], ["-force-attribute=alwaysinline"]):
+        _run([LLVM_BIN / "opt", "-passes=internalize,globaldce,default<O3>", f"-internalize-public-api-list={KERNEL_SYMBOL}",
+              *forced, bitcode, "-o", optimised], "link.optimise")
+        _run([LLVM_BIN / "clang", "-x", "ir", "-target", "amdgcn-amd-amdhsa", f"-mcpu={arch}", "-O3", "-nogpulib",
+              optimised, "-o", hsaco], "link.codegen")
+        text = _run([LLVM_BIN / "llvm-objdump", "-d", "--no-show-raw-insn", hsaco], "audit.disassemble")
+        if not re.search(r"\bs_swappc_b64\b|\bs_setpc_b64\b", text):
+            break
 
 
 def audit(hsaco: Path) -> dict[str, int]:

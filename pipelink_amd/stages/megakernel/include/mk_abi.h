@@ -46,7 +46,7 @@ typedef struct MkModel {
   uint16_t* kv_cache;      /* bf16 [L][2][SMAX][HKV][64] */
   float* x;                /* [D] residual stream, in and out */
   float* qkv;              /* [(HQ + 2 HKV) * 64] */
-  float* attn_partial;     /* [HQ][chunks][64 + 2]: unnormalised output, running maximum (log2 units), sum */
+  float* attn_partial;     /* [HQ][chunks][MK_PARTIAL_STRIDE]: unnormalised output, maximum (log2 units), sum */
   float* h;                /* [DFF] */
   float* logits;           /* [V] */
   const float* rope;       /* [2][32]: cos, sin of pos * theta^(-2 i / 64) */

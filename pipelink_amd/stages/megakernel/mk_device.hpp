@@ -55,9 +55,36 @@ __device__ __forceinline__ void my_rows(int total, int& first, int& last) {
   last = min(first + per, total);
 }
 
+// Lane exchanges inside a row of 16 lanes as DPP operands of the add itself (no LDS round trip as a shuffle is):
+// 0xB1 / 0x4E swap neighbours / pairs inside a quad, 0x141 mirrors each half row (swaps its quads), 0x140 mirrors
+// the row (swaps its halves), 0x104 reads the lane four further on, 0x128 the lane eight away.
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+// sum over the wave, in every lane
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int s = 32; s >= 1; s >>= 1) v += __shfl_xor(v, s);
+  v += dpp<0xB1>(v);
+  v += dpp<0x4E>(v);
+  v += dpp<0x141>(v);
+  v += dpp<0x140>(v);  // every lane: the sum of its row
+  return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp<0xB1>(v));
+  v = fmaxf(v, dpp<0x4E>(v));
+  v = fmaxf(v, dpp<0x141>(v));
+  v = fmaxf(v, dpp<0x140>(v));
+  return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
+}
+// sum over each aligned group of eight lanes, valid in the group's first lane
+__device__ __forceinline__ float sum8_first(float v) {
+  v += dpp<0xB1>(v);
+  v += dpp<0x4E>(v);
+  v += dpp<0x104>(v);
   return v;
 }
 
@@ -70,50 +97,85 @@ __device__ __forceinline__ float dot8(const v4i w, const v4f x0, const v4f x1) {
   return acc;
 }
 
-// Dots of R consecutive bf16 rows (n elements each, n % 512 == 0, `pitch` elements apart) with the fp32 vector in
-// LDS, by one wave: all R x 4 loads of a pass are issued before any is used, so a lane keeps up to 4 R sixteen-byte
-// loads in flight.  Every lane gets the sums.
+// One pass over R consecutive bf16 rows (`pitch` elements apart, n elements each, n % 8 == 0): lane `c0` takes the
+// 8-element chunks c0, c0 + 64, c0 + 128, c0 + 192 of every row.  rows_load issues the R x 4 sixteen-byte loads,
+// rows_fma uses them against the fp32 vector in LDS: between the two a caller can do what does not need them.
 template <int R>
-__device__ __forceinline__ void rows_dot(const uint16_t* rows, int64_t pitch, const float* x, int n, int lane, float (&sum)[R]) {
-  float acc[R];
+__device__ __forceinline__ void rows_load(const uint16_t* rows, int64_t pitch, int n, int c0, v4i (&w)[R][4]) {
 #pragma unroll
-  for (int r = 0; r < R; ++r) acc[r] = 0.0f;
-  for (int c0 = lane; c0 < n / 8; c0 += 256) {  // four chunks of 8 elements per lane and pass
-    v4i w[R][4];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const v4i zero = {0, 0, 0, 0};
-        w[r][j] = c0 + 64 * j < n / 8 ? *reinterpret_cast<const v4i*>(rows + r * pitch + 8 * (c0 + 64 * j)) : zero;
-      }
+  for (int r = 0; r < R; ++r)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      if (c0 + 64 * j >= n / 8) break;  // rows shorter than 2048 elements
-      const v4f x0 = *reinterpret_cast<const v4f*>(x + 8 * (c0 + 64 * j)), x1 = *reinterpret_cast<const v4f*>(x + 8 * (c0 + 64 * j) + 4);
-#pragma unroll
-      for (int r = 0; r < R; ++r) acc[r] += dot8(w[r][j], x0, x1);
+      const v4i zero = {0, 0, 0, 0};
+      w[r][j] = c0 + 64 * j < n / 8 ? *reinterpret_cast<const v4i*>(rows + r * pitch + 8 * (c0 + 64 * j)) : zero;
     }
+}
+template <int R>
+__device__ __forceinline__ void rows_fma(const v4i (&w)[R][4], const float* x, int n, int c0, float (&acc)[R]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (c0 + 64 * j >= n / 8) break;  // rows shorter than 2048 elements
+    const v4f x0 = *reinterpret_cast<const v4f*>(x + 8 * (c0 + 64 * j)), x1 = *reinterpret_cast<const v4f*>(x + 8 * (c0 + 64 * j) + 4);
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] += dot8(w[r][j], x0, x1);
   }
+}
+template <int R>
+__device__ __forceinline__ void wave_sums(float (&acc)[R]) {
 #pragma unroll
-  for (int s = 32; s >= 1; s >>= 1)
-#pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] += __shfl_xor(acc[r], s);
-#pragma unroll
-  for (int r = 0; r < R; ++r) sum[r] = acc[r];
+  for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
 }
 
-// y(row) for this workgroup's rows [first, last) of a matrix with rows of n elements: waves take groups of R rows
+// Dots of R consecutive bf16 rows with the fp32 vector in LDS, by one wave; every lane gets the sums.  `first` holds
+// the loads of the first pass (c0 = lane) if the caller issued them already.
+template <int R>
+__device__ __forceinline__ void rows_dot(const uint16_t* rows, int64_t pitch, const float* x, int n, int lane, float (&sum)[R],
+                                         const v4i (*first)[R][4] = nullptr) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) sum[r] = 0.0f;
+  int c0 = lane;
+  if (first) {
+    rows_fma<R>(*first, x, n, c0, sum);
+    c0 += 256;
+  }
+  for (; c0 < n / 8; c0 += 256) {
+    v4i w[R][4];
+    rows_load<R>(rows, pitch, n, c0, w);
+    rows_fma<R>(w, x, n, c0, sum);
+  }
+  wave_sums<R>(sum);
+}
+
+// y(row) for this workgroup's rows [first, last) of a matrix with rows of n elements: waves take groups of R rows.
+// Rows of up to 2048 elements are one pass each, and then a wave loads its next group before it sums the present one.
 template <int R, typename Emit>
 __device__ __forceinline__ void matvec(const uint16_t* w, int n, const float* x, int first, int last, Emit&& emit) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int r = first + R * wave;
-  for (; r + R <= last; r += 4 * R) {
+  auto finish = [&](const v4i (&loaded)[R][4], int row) {
     float sum[R];
-    rows_dot<R>(w + (int64_t)r * n, n, x, n, lane, sum);
+    rows_dot<R>(w + (int64_t)row * n, n, x, n, lane, sum, &loaded);
     if (lane == 0) {
 #pragma unroll
-      for (int i = 0; i < R; ++i) emit(r + i, sum[i]);
+      for (int i = 0; i < R; ++i) emit(row + i, sum[i]);
+    }
+  };
+  if (r + R <= last) {
+    v4i wa[R][4], wb[R][4];
+    rows_load<R>(w + (int64_t)r * n, n, n, lane, wa);
+    for (;;) {
+      int next = r + 4 * R;
+      bool more = next + R <= last;
+      if (more) rows_load<R>(w + (int64_t)next * n, n, n, lane, wb);
+      finish(wa, r);
+      r = next;
+      if (!more) break;
+      next = r + 4 * R;
+      more = next + R <= last;
+      if (more) rows_load<R>(w + (int64_t)next * n, n, n, lane, wa);
+      finish(wb, r);
+      r = next;
+      if (!more) break;
     }
   }
   for (; r < last; ++r) {  // a last group with fewer than R rows
@@ -122,14 +184,20 @@ __device__ __forceinline__ void matvec(const uint16_t* w, int n, const float* x,
     if (lane == 0) emit(r, sum[0]);
   }
 }
-// y(row) for R consecutive rows (R <= 8): the four waves take a quarter of the columns each (n % 2048 == 0 or the
-// quarter is a multiple of 512), so that R x 4 loads per lane are in flight on every wave; partial sums meet in
-// `scratch` (4 x R floats of LDS).  All threads must call it; ends with a barrier-protected emit by threads < R.
+// y(row) for R consecutive rows (R <= 8) by the whole workgroup: the four waves take a quarter of the columns each
+// (n % 32 == 0), so that R x 4 loads per lane are in flight on every wave; the partial sums meet in `scratch`
+// (4 x R floats of LDS).  split_load issues a wave's first pass; matvec_split (all threads call it) does the rest
+// and ends with threads < count emitting one row each.
+template <int R>
+__device__ __forceinline__ void split_load(const uint16_t* rows, int n, v4i (&w)[R][4]) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  rows_load<R>(rows + wave * (n / 4), n, n / 4, lane, w);
+}
 template <int R, typename Emit>
-__device__ __forceinline__ void matvec_split(const uint16_t* rows, int n, const float* x, float* scratch, int count, Emit&& emit) {
+__device__ __forceinline__ void matvec_split(const uint16_t* rows, int n, const float* x, float* scratch, int count, const v4i (&loaded)[R][4], Emit&& emit) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, q = n / 4;
   float sum[R];
-  rows_dot<R>(rows + wave * q, n, x + wave * q, q, lane, sum);
+  rows_dot<R>(rows + wave * q, n, x + wave * q, q, lane, sum, &loaded);
   if (lane == 0) {
 #pragma unroll
     for (int i = 0; i < R; ++i) scratch[wave * R + i] = sum[i];

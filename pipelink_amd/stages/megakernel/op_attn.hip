@@ -22,43 +22,58 @@ extern "C" __device__ void mk_attn_op(const void* view, const MkInstr* instr) {
   if (head >= m.hq) return;
   const int kvh = head / (m.hq / m.hkv);
   const int npos = m.pos + 1;  // the cache holds positions 0 .. pos - 1, the step's own token is position pos
-  const int per = (npos + m.chunks - 1) / m.chunks;
-  const int p0 = min(chunk * per, npos), p1 = min(p0 + per, npos);
+  // the cached positions are dealt evenly to the chunks; the last chunk takes the step's own token as well
+  const int per = (m.pos + m.chunks - 1) / m.chunks;
+  const int p0 = min(chunk * per, m.pos), p1 = chunk == m.chunks - 1 ? npos : min(p0 + per, m.pos);
   float* q = mk::vec();            // [64] rotated query
   float* knew = q + 64;            // [64] the step's rotated key, rounded to bf16 as the cache will hold it
   float* red = q + 128;            // [8] reduction scratch
-  float* part = q + 256;           // [4][64] per-wave partial outputs
-  float* score = q + 512;          // [per]
+  float* part = q + 256;           // [16][64] partial outputs, one per row of 16 lanes
+  float* score = q + 1280;         // [per + 1]
   const uint16_t* kc = m.kv_cache + (((int64_t)instr->layer * 2 + 0) * m.smax * m.hkv + kvh) * MK_HEAD_DIM;
   const uint16_t* vc = m.kv_cache + (((int64_t)instr->layer * 2 + 1) * m.smax * m.hkv + kvh) * MK_HEAD_DIM;
   const int64_t pos_stride = (int64_t)m.hkv * MK_HEAD_DIM;
   const float* vnew = m.qkv + (m.hq + m.hkv + kvh) * MK_HEAD_DIM;
+  // Eight lanes take one position (eight elements each, one 16-byte load), a wave eight positions per load
+  // instruction, the workgroup 32.  The first sixteen such loads of the keys and of the values (512 positions) are
+  // asked for before the query is rotated: neither depends on it.
+  constexpr int AHEAD = 16;
+  const int cached_end = min(p1, m.pos), last_cached = max(m.pos - 1, 0);
+  const int g = lane >> 3, piece = lane & 7, pl0 = p0 + 8 * wave + g;
+  mk::v4i kreg[AHEAD], vreg[AHEAD];
+#pragma unroll
+  for (int j = 0; j < AHEAD; ++j) kreg[j] = *reinterpret_cast<const mk::v4i*>(kc + min(pl0 + 32 * j, last_cached) * pos_stride + 8 * piece);
+#pragma unroll
+  for (int j = 0; j < AHEAD; ++j) vreg[j] = *reinterpret_cast<const mk::v4i*>(vc + min(pl0 + 32 * j, last_cached) * pos_stride + 8 * piece);
   if (tid < 64) q[tid] = pipelink_call_rope_apply(view, m.qkv + head * MK_HEAD_DIM, tid);
   else if (tid < 128) knew[tid - 64] = mk_attn::bf16_round(pipelink_call_rope_apply(view, m.qkv + (m.hq + kvh) * MK_HEAD_DIM, tid - 64));
   __syncthreads();
   // ---- scores (log2 units) and the chunk's maximum ---------------------------------------------------------
   float local_max = -1.0e30f;
-  for (int p = p0 + tid; p < p1; p += MK_THREADS) {
-    float s = 0.0f;
-    if (p < m.pos) {
-      const mk::v4i* row = reinterpret_cast<const mk::v4i*>(kc + p * pos_stride);
+  {
+    const mk::v4f q0 = *reinterpret_cast<const mk::v4f*>(q + 8 * piece), q1 = *reinterpret_cast<const mk::v4f*>(q + 8 * piece + 4);
+    for (int pb = pl0; pb < cached_end; pb += 32 * AHEAD) {
+      if (pb != pl0) {
 #pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        const mk::v4i w = row[c];
-        const uint32_t u[4] = {(uint32_t)w.x, (uint32_t)w.y, (uint32_t)w.z, (uint32_t)w.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          s += mk::bf16_to_f32(u[e] & 0xFFFFu) * q[8 * c + 2 * e] + __uint_as_float(u[e] & 0xFFFF0000u) * q[8 * c + 2 * e + 1];
+        for (int j = 0; j < AHEAD; ++j) kreg[j] = *reinterpret_cast<const mk::v4i*>(kc + min(pb + 32 * j, last_cached) * pos_stride + 8 * piece);
       }
-    } else {
-      for (int i = 0; i < 64; ++i) s += knew[i] * q[i];
-    }
-    s *= m.attn_scale_log2e;
-    score[p - p0] = s;
-    local_max = fmaxf(local_max, s);
-  }
 #pragma unroll
-  for (int sh = 32; sh >= 1; sh >>= 1) local_max = fmaxf(local_max, __shfl_xor(local_max, sh));
+      for (int j = 0; j < AHEAD; ++j) {
+        const float sc = mk::sum8_first(mk::dot8(kreg[j], q0, q1)) * m.attn_scale_log2e;
+        const int p = pb + 32 * j;
+        if (p < cached_end && piece == 0) {
+          score[p - p0] = sc;
+          local_max = fmaxf(local_max, sc);
+        }
+      }
+    }
+    if (p0 <= m.pos && m.pos < p1 && wave == 0) {  // the step's own token
+      const float sc = mk::wave_sum(knew[lane] * q[lane]) * m.attn_scale_log2e;
+      if (lane == 0) score[m.pos - p0] = sc;
+      local_max = fmaxf(local_max, sc);
+    }
+  }
+  local_max = mk::wave_max(local_max);
   if (lane == 0) red[wave] = local_max;
   __syncthreads();
   const float cmax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
@@ -71,44 +86,47 @@ extern "C" __device__ void mk_attn_op(const void* view, const MkInstr* instr) {
   local_sum = mk::wave_sum(local_sum);
   if (lane == 0) red[4 + wave] = local_sum;
   __syncthreads();
-  // ---- unnormalised output: 16 lanes take one position (four d each, one 8-byte load), a wave four positions per
-  // load instruction and sixteen such loads in flight ------------------------------------------------------
+  // ---- unnormalised output -----------------------------------------------------------------------------------
   {
-    const int g = lane >> 4, dq = lane & 15;
-    const int cached_end = min(p1, m.pos), last_cached = max(m.pos - 1, 0);
-    float o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int pb = p0 + 4 * wave + g; pb < cached_end; pb += 16 * 16) {
-      uint2 v[16];
+    float o[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    for (int pb = pl0; pb < cached_end; pb += 32 * AHEAD) {
+      if (pb != pl0) {
 #pragma unroll
-      for (int j = 0; j < 16; ++j) v[j] = *reinterpret_cast<const uint2*>(vc + min(pb + 16 * j, last_cached) * pos_stride + 4 * dq);
+        for (int j = 0; j < AHEAD; ++j) vreg[j] = *reinterpret_cast<const mk::v4i*>(vc + min(pb + 32 * j, last_cached) * pos_stride + 8 * piece);
+      }
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const int p = pb + 16 * j;
-        const float s = p < cached_end ? score[p - p0] : 0.0f;
-        o[0] += s * mk::bf16_to_f32(v[j].x & 0xFFFFu);
-        o[1] += s * __uint_as_float(v[j].x & 0xFFFF0000u);
-        o[2] += s * mk::bf16_to_f32(v[j].y & 0xFFFFu);
-        o[3] += s * __uint_as_float(v[j].y & 0xFFFF0000u);
+      for (int j = 0; j < AHEAD; ++j) {
+        const int p = pb + 32 * j;
+        const float sc = p < cached_end ? score[p - p0] : 0.0f;
+        const uint32_t u[4] = {(uint32_t)vreg[j].x, (uint32_t)vreg[j].y, (uint32_t)vreg[j].z, (uint32_t)vreg[j].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          o[2 * e] += sc * mk::bf16_to_f32(u[e] & 0xFFFFu);
+          o[2 * e + 1] += sc * __uint_as_float(u[e] & 0xFFFF0000u);
+        }
       }
     }
     if (p0 <= m.pos && m.pos < p1 && wave == 0 && g == 0) {  // the step's own token, as the cache will hold it
-      const float s = score[m.pos - p0];
+      const float sc = score[m.pos - p0];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] += s * mk_attn::bf16_round(mk::shared_load(vnew + 4 * dq + e));
+      for (int e = 0; e < 8; ++e) o[e] += sc * mk_attn::bf16_round(mk::shared_load(vnew + 8 * piece + e));
     }
+    // the row's two groups of eight lanes together (every lane takes part in the exchange), then one partial output per row
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      o[e] += __shfl_xor(o[e], 16);
-      o[e] += __shfl_xor(o[e], 32);
-    }
-    if (g == 0) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) part[wave * 64 + 4 * dq + e] = o[e];
+    for (int e = 0; e < 8; ++e) o[e] += mk::dpp<0x128>(o[e]);
+    if ((lane & 8) == 0) {
+      *reinterpret_cast<mk::v4f*>(part + (4 * wave + (lane >> 4)) * 64 + 8 * piece) = mk::v4f{o[0], o[1], o[2], o[3]};
+      *reinterpret_cast<mk::v4f*>(part + (4 * wave + (lane >> 4)) * 64 + 8 * piece + 4) = mk::v4f{o[4], o[5], o[6], o[7]};
     }
   }
   __syncthreads();
   float* out = m.attn_partial + ((int64_t)head * m.chunks + chunk) * MK_PARTIAL_STRIDE;
-  if (tid < 64) mk::shared_store(out + tid, part[tid] + part[64 + tid] + part[128 + tid] + part[192 + tid]);
+  if (tid < 64) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int row = 0; row < 16; ++row) sum += part[64 * row + tid];
+    mk::shared_store(out + tid, sum);
+  }
   if (tid == 64) {
     mk::shared_store(out + MK_HEAD_DIM, cmax);
     mk::shared_store(out + MK_HEAD_DIM + 1, red[4] + red[5] + red[6] + red[7]);

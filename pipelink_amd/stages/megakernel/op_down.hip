@@ -7,20 +7,30 @@
 extern "C" __device__ void mk_down_op(const void* view, const MkInstr* instr) {
   const MkModel& m = mk::model(view);
   float* hv = mk::vec();
-  for (int i = 4 * threadIdx.x; i < m.dff; i += 4 * MK_THREADS) *reinterpret_cast<mk::v4f*>(hv + i) = mk::shared_load4(m.h, i, m.dff);
-  __syncthreads();
-  const uint16_t* w = mk::layer_of(m, instr->layer).wdown;
   float* scratch = hv + 8192;  // behind the vector
+  const uint16_t* w = mk::layer_of(m, instr->layer).wdown;
   int first, last;
   mk::my_rows(m.d, first, last);
-  for (int r = first; r < last; r += 8) {
-    const int count = min(8, last - r);
-    if (count == 8) {
-      mk::matvec_split<8>(w + (int64_t)r * m.dff, m.dff, hv, scratch, 8, [&](int i, float v) { mk::shared_store(m.x + r + i, mk::shared_load(m.x + r + i) + v); });
-    } else {
-      mk::matvec<1>(w, m.dff, hv, r, last, [&](int row, float v) { mk::shared_store(m.x + row, mk::shared_load(m.x + row) + v); });
+  // the intermediate, this workgroup's first eight rows of the matrix and the residual they add to: all on their way at once
+  mk::v4f hreg[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) hreg[j] = mk::shared_load4(m.h, 4 * (int)threadIdx.x + 4 * MK_THREADS * j, m.dff);  // past DFF: zeros
+  mk::v4i wreg[8][4];
+  if (first + 8 <= last) mk::split_load<8>(w + (int64_t)first * m.dff, m.dff, wreg);
+  float xold = (int)threadIdx.x < 8 && first + (int)threadIdx.x < last ? mk::shared_load(m.x + first + threadIdx.x) : 0.0f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    if (4 * (int)threadIdx.x + 4 * MK_THREADS * j < m.dff) *reinterpret_cast<mk::v4f*>(hv + 4 * threadIdx.x + 4 * MK_THREADS * j) = hreg[j];
+  __syncthreads();
+  int r = first;
+  for (; r + 8 <= last; r += 8) {
+    if (r != first) {
+      mk::split_load<8>(w + (int64_t)r * m.dff, m.dff, wreg);
+      xold = (int)threadIdx.x < 8 ? mk::shared_load(m.x + r + threadIdx.x) : 0.0f;
     }
+    mk::matvec_split<8>(w + (int64_t)r * m.dff, m.dff, hv, scratch, 8, wreg, [&](int i, float v) { mk::shared_store(m.x + r + i, xold + v); });
   }
+  mk::matvec<1>(w, m.dff, hv, r, last, [&](int row, float v) { mk::shared_store(m.x + row, mk::shared_load(m.x + row) + v); });
 }
 #else
 #include "include/mk_abi.h"
