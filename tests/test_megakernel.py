@@ -149,6 +149,11 @@ def test_stated_model_against_the_oracle_and_its_time_per_token():
     bytes_per_token = weights.numel() * 2 + cache[:, :, :4096].numel() * 2
     print(f"decode step: {got['ms']:.3f} ms per token, {bytes_per_token / got['ms'] / 1e9:.2f} TB/s of {bytes_per_token / 1e9:.2f} GB "
           f"(weights + cache read once), {bytes_per_token / got['ms'] / 1e9 / 8 * 100:.1f} % of 8 TB/s", flush=True)
+    control = _run("link_json", cfg, weights, cache, x, workgroups=256, image_key="one_unit", time_launches=20)
+    assert all(np.array_equal(control[n], got[n]) for n in ("logits", "x", "kv_cache")), "linked and one-unit images differ"
+    ratio = control["ms"] / got["ms"]
+    print(f"one-unit control: {control['ms']:.3f} ms per token; linked / one-unit throughput ratio {ratio:.4f}", flush=True)
+    assert ratio >= 0.97                                   # the seam gate of campaigns/megakernel/evidence/RESULT.md:7
     swapped = _run("swap_link_json", cfg, weights, cache, x, workgroups=256, time_launches=20)
     assert _rel(swapped["logits"], got["logits"]) <= 1e-4
     print(f"with mk.attn.wide relinked: {swapped['ms']:.3f} ms per token", flush=True)
