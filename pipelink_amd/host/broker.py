@@ -5,15 +5,18 @@ Plays the part of ``pipec2.host.broker.open_host`` (pipec/src/pipec2/host/broker
 the routed-expert FFN pipeline: the owners' providers (``pipelink_params_{abi,query,build,
 release}_<suffix>``, include/plk_host_abi_v2.h) live in the C-ABI library; the broker owns every
 record, array and the residue bytes, checks each provider's answers against what the caller
-holds, and releases sessions in reverse build order (broker.py:768-801).  What the reference
-reads from the ``host`` section of link.json (owner inventory, channel lists) is the table
-``OWNERS`` here -- the three owners and their channels are fixed for this pipeline.
+holds, and releases sessions in reverse build order (broker.py:768-801).  The owner inventory
+comes from the ``host`` section of link.json (broker.py:818-830): per params group the provider's
+entry points, the record types it must report, its scalars and its caller-owned channels with
+their extents as expressions over the scalars -- the stages declared them (``PL_HOST_*``), the
+link gathered them.  This side only keeps the ctypes mirrors of the record types, by C name.
 
 Pure ctypes; nothing here needs a GPU until ``HostSession.launch``."""
 from __future__ import annotations
 
 import ctypes
 import hashlib
+import re
 import struct
 from ctypes import (POINTER, Structure, byref, c_int64, c_size_t, c_uint8, c_uint32, c_uint64, c_void_p, cast, pointer,
                     sizeof)
@@ -169,38 +172,44 @@ NEUTRAL_TYPES = [
     (0x70000014, "plk_domain_v2", Domain),
 ]
 
-# scalar ids (include/plk_host_abi_v2.h)
-SCALARS = {"mok.num_local_tokens": 1, "mok.hidden": 2, "mok.intermediate": 3, "mok.num_local_experts": 4,
-           "mok.swiglu_limit": 10, "mok.pass": 11, "mok.precision": 12, "mok.routed_rows": 60, "mok.ld_q_h": 61,
-           "mok.ld_q_i": 62, "mok.ld_sc_h": 63, "mok.ld_sc_i": 64}
+# ctypes mirrors of the owner-local record types a link may name (C name -> mirror)
+MIRRORS = {"MokGemmResidue": MokGemmResidue, "MokActResidue": MokActResidue, "MokFrameworkParams": MokFrameworkParams,
+           "MokMxView": MokMxView}
+_TERM = re.compile(r"^(?:(\d+)|([A-Za-z_][\w.]*)|(floor|ceil)\(([A-Za-z_][\w.]*),(\d+)\))$")
 
 
-def _shapes(s: Mapping[str, int]) -> dict[str, dict[str, tuple[int, int, tuple[int, ...]]]]:
-    """(element bits, access, extents) of every channel of every owner for the given scalars."""
-    t, h, i, e, r = (s[k] for k in ("mok.num_local_tokens", "mok.hidden", "mok.intermediate", "mok.num_local_experts",
-                                    "mok.routed_rows"))
-    wq = lambda n, k: (8, ACCESS_READ, (e, k // 64, n, 64))
-    wsc = lambda n, k: (8, ACCESS_READ, (e, (k + 127) // 128, n, 4))
-    return {
-        "mok.framework": {"tokens_per_expert": (32, ACCESS_READ, (e,))},
-        "mok.gemm": {
-            "x_q": (8, ACCESS_READ, (t, s["mok.ld_q_h"])), "x_sc": (8, ACCESS_READ, (t, s["mok.ld_sc_h"])),
-            "w_gate_q": wq(i, h), "w_gate_sc": wsc(i, h), "w_up_q": wq(i, h), "w_up_sc": wsc(i, h),
-            "w_down_q": wq(h, i), "w_down_sc": wsc(h, i),
-            "hidden_q": (8, ACCESS_READ, (r, s["mok.ld_q_i"])), "hidden_sc": (8, ACCESS_READ, (r, s["mok.ld_sc_i"])),
-            "y": (16, ACCESS_WRITE, (r, h)), "row_token": (32, ACCESS_READ, (r,)),
-        },
-        "mok.act": {"hidden_q": (8, ACCESS_WRITE, (r, s["mok.ld_q_i"])), "hidden_sc": (8, ACCESS_WRITE, (r, s["mok.ld_sc_i"]))},
-    }
+def host_inventory(link: Mapping[str, Any]) -> dict[str, Any]:
+    """link.json["host"], or the failure the reference's broker raises without one (broker.py:818-820)."""
+    host = link.get("host")
+    if not host or host.get("protocol") != 2:
+        raise PlkError(4, "link.host: a link with a host section (protocol 2) is required")
+    return host
 
 
-# stage id -> (entry point suffix, owner-local types it reports: (id, C name, mirror))
-OWNERS = {
-    "mok.framework": ("mok_framework", [(3, "MokFrameworkParams", MokFrameworkParams)]),
-    "mok.gemm": ("mok_gemm", [(1, "MokGemmResidue", MokGemmResidue), (4, "MokMxView", MokMxView)]),
-    "mok.act": ("mok_act", [(2, "MokActResidue", MokActResidue)]),
-}
-OPTIONAL = {("mok.gemm", "row_token")}
+def evaluate_extents(text: str, scalars: Mapping[str, Any]) -> tuple[int, ...]:
+    """A channel's extents: comma-separated integers, scalar names, floor(name,int) or ceil(name,int)."""
+    out = []
+    for term in re.findall(r"(?:floor|ceil)\([^)]*\)|[^,]+", text.replace(" ", "")):
+        m = _TERM.match(term)
+        if not m:
+            raise PlkError(4, f"link.host: cannot read the extent term {term!r}")
+        if m.group(1):
+            out.append(int(m.group(1)))
+            continue
+        name = m.group(2) or m.group(4)
+        if name not in scalars:
+            raise PlkError(3, f"scalar {name} is missing")
+        value = int(scalars[name])
+        out.append(value if m.group(2) else value // int(m.group(5)) if m.group(3) == "floor" else -(-value // int(m.group(5))))
+    return tuple(out)
+
+
+def channel_shapes(link: Mapping[str, Any], scalars: Mapping[str, Any]) -> dict[str, dict[str, tuple[int, int, tuple[int, ...]]]]:
+    """owner -> channel name -> (element bits, access, extents) for the given scalars, channels in id order."""
+    access = {"read": ACCESS_READ, "write": ACCESS_WRITE}
+    return {g["owner"]: {c["name"]: (c["elem_bits"], access[c["access"]], evaluate_extents(c["extents"], scalars))
+                         for c in sorted(g["channels"], key=lambda c: c["id"])}
+            for g in host_inventory(link)["groups"]}
 
 
 def layout_digest(name: str, mirror: type[Structure]) -> bytes:
@@ -231,17 +240,18 @@ def _check(status: int, what: str) -> None:
 class _Scalars:
     """The shared scalar image: header, then plk_scalar_v2 records (device-safe: offsets, no pointers)."""
 
-    def __init__(self, values: Mapping[str, Any]):
-        unknown = set(values) - set(SCALARS)
+    def __init__(self, values: Mapping[str, Any], declared: list[Mapping[str, Any]]):
+        ids = {d["name"]: d for d in declared}
+        unknown = set(values) - set(ids)
         if unknown:
             raise PlkError(3, f"unknown scalars {sorted(unknown)}")
         recs = b""
-        for name in sorted(values, key=SCALARS.get):
+        for name in sorted(values, key=lambda n: ids[n]["id"]):
             v = values[name]
-            if name == "mok.swiglu_limit":
-                recs += struct.pack("<IIQ", SCALARS[name], SCALAR_F64, struct.unpack("<Q", struct.pack("<d", float(v)))[0])
+            if ids[name]["kind"] == "f64":
+                recs += struct.pack("<IIQ", ids[name]["id"], SCALAR_F64, struct.unpack("<Q", struct.pack("<d", float(v)))[0])
             else:
-                recs += struct.pack("<IIq", SCALARS[name], SCALAR_I64, int(v))
+                recs += struct.pack("<IIq", ids[name]["id"], SCALAR_I64, int(v))
         head = SharedScalars(Header(ABI_V2, sizeof(SharedScalars)), sizeof(SharedScalars) + len(recs), len(values), sizeof(SharedScalars))
         self.buffer = ctypes.create_string_buffer(bytes(head) + recs, sizeof(SharedScalars) + len(recs))
         self.pointer = cast(self.buffer, POINTER(SharedScalars))
@@ -250,13 +260,20 @@ class _Scalars:
 class Owner:
     """One params group: its provider's four entry points and the records exchanged with it."""
 
-    def __init__(self, lib: ctypes.CDLL, stage_id: str):
-        self.stage_id = stage_id
-        suffix, self.local_types = OWNERS[stage_id]
-        self.abi = getattr(lib, f"pipelink_params_abi_{suffix}")
-        self.query = getattr(lib, f"pipelink_params_query_{suffix}")
-        self.build = getattr(lib, f"pipelink_params_build_{suffix}")
-        self.release = getattr(lib, f"pipelink_params_release_{suffix}")
+    def __init__(self, lib: ctypes.CDLL, group: Mapping[str, Any]):
+        self.group, self.stage_id = group, group["owner"]
+        self.local_types = []
+        for t in group["provider"]["abi_types"]:
+            mirror = MIRRORS.get(t["name"])
+            if mirror is None or sizeof(mirror) != t["bytes"] or ctypes.alignment(mirror) != t["align"]:
+                raise PlkError(1, f"{self.stage_id}: the link declares {t['name']} ({t['bytes']} bytes, align {t['align']}), "
+                                  "which this broker does not mirror")
+            self.local_types.append((t["id"], t["name"], mirror))
+        symbols = group["provider"]["symbols"]
+        try:
+            self.abi, self.query, self.build, self.release = (getattr(lib, symbols[k]) for k in ("abi", "query", "build", "release"))
+        except AttributeError as err:
+            raise PlkError(4, f"{self.stage_id}: missing provider export: {err}") from None
         self.abi.argtypes, self.abi.restype = [POINTER(AbiReport)], ctypes.c_int
         self.query.argtypes, self.query.restype = [POINTER(Common), c_void_p, POINTER(Demands)], ctypes.c_int
         self.build.argtypes = [POINTER(Common), c_void_p, POINTER(Resources), c_void_p, c_size_t, POINTER(TransferReport),
@@ -332,27 +349,31 @@ def plan(link: Mapping[str, Any], resources: Mapping[str, Mapping[str, Resource]
 
     Host-only: touches no device memory.  ``resources`` maps stage id -> channel name -> Resource."""
     lib = lib or load_library()
+    host = host_inventory(link)
+    groups = {g["owner"]: g for g in host["groups"]}
     entries = {e["stage_id"]: e for e in link["params"]["entries"]}
-    if set(entries) != set(OWNERS) or set(resources) != set(OWNERS):
-        raise PlkError(4, "link.json params entries and resources must name exactly the pipeline's owners")
-    missing = set(SCALARS) - set(scalars)
+    blobs = {b["stage_id"] for b in host["params"]["blobs"] if b["bytes"]}
+    if set(entries) - blobs != set(groups) or set(resources) != set(groups):
+        raise PlkError(4, "link.json params entries and resources must name exactly the link's owners")
+    missing = {d["name"] for d in host["scalars"]} - set(scalars)
     if missing:
         raise PlkError(3, f"scalars {sorted(missing)} are missing")
-    shapes = _shapes(scalars)
-    shared = _Scalars(scalars)
+    shapes = channel_shapes(link, scalars)
+    optional = {(g["owner"], c["name"]) for g in host["groups"] for c in g["channels"] if c["optional"]}
+    shared = _Scalars(scalars, host["scalars"])
     block = Dim3(link["threads"], 1, 1)
     image = bytearray(link["params"]["total_bytes"])
     geometry: dict[str, Any] = {}
     owners: list[Owner] = []
     keep: list[Any] = [shared]
     try:
-        for stage_id in (s["stage_id"] for s in link["params"]["entries"]):
-            owner = Owner(lib, stage_id)
+        for stage_id in (s["stage_id"] for s in link["params"]["entries"] if s["stage_id"] in groups):
+            owner = Owner(lib, groups[stage_id])
             owners.append(owner)
             rep = owner.report()
             names = list(shapes[stage_id])
             if set(resources[stage_id]) - set(names) or \
-                    {n for n in names if (stage_id, n) not in OPTIONAL} - set(resources[stage_id]):
+                    {n for n in names if (stage_id, n) not in optional} - set(resources[stage_id]):
                 raise PlkError(4, f"{stage_id}: resources must cover channels {names}")
             n = len(names)
             metas, demands = (TensorMeta * n)(), (ChannelDemand * n)()

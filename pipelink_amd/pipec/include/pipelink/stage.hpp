@@ -161,6 +161,25 @@ inline int emit_main() {
                                ::pl::quote(result) + ",\"dtype\":" + ::pl::quote(dtype) + ",\"shape\":[" + ::pl::num(rows) + \
                                "," + ::pl::num(cols) + "],\"layout\":" + ::pl::quote(layout) + "}")
 // a published geometry fact of this owner (reaches other owners only through the link)
+// ---- host contract: what the broker needs to know to build this stage's params through a provider library
+// (the reference's PL_HOST_GROUP / PL_HOST_ABI_* / PL_HOST_SCALARS / PL_HOST_CHANNEL, pack/include/pipelink/host.hpp).
+// The link gathers these into link.json["host"]["groups"].
+// the params group and the suffix of the provider's four entry points pipelink_params_{abi,query,build,release}_<suffix>
+#define PL_HOST_GROUP(params_group, provider_suffix) \
+  PL_REG("host_group", "{\"params_group\":" + ::pl::quote(params_group) + ",\"provider\":" + ::pl::quote(provider_suffix) + "}")
+// an owner-local record type the provider reports: its id, and what this compiler makes of it
+#define PL_HOST_ABI_TYPE(id, T) \
+  PL_REG("host_types", "{\"id\":" + ::pl::num(id) + ",\"name\":" + ::pl::quote(#T) + ",\"bytes\":" + ::pl::num(sizeof(T)) + \
+                           ",\"align\":" + ::pl::num(alignof(T)) + "}")
+// a scalar of the shared scalar image: kind "i64" or "f64"
+#define PL_HOST_SCALAR(id, name, kind) \
+  PL_REG("host_scalars", "{\"id\":" + ::pl::num(id) + ",\"name\":" + ::pl::quote(name) + ",\"kind\":" + ::pl::quote(kind) + "}")
+// a caller-owned tensor: channel id, caller's name, element bits, "read" or "write", extents as a comma-separated
+// list of terms (an integer, a scalar name, floor(name,int) or ceil(name,int)), and whether the caller may leave it out
+#define PL_HOST_CHANNEL(id, name, elem_bits, access, extents, optional)                                                      \
+  PL_REG("host_channels", "{\"id\":" + ::pl::num(id) + ",\"name\":" + ::pl::quote(name) + ",\"elem_bits\":" +             \
+                              ::pl::num(elem_bits) + ",\"access\":" + ::pl::quote(access) + ",\"extents\":" +              \
+                              ::pl::quote(extents) + ",\"optional\":" + ((optional) ? "true" : "false") + "}")
 #define PL_FACT(name, value) PL_REG("facts", "{\"name\":" + ::pl::quote(name) + ",\"value\":" + ::pl::num(value) + "}")
 // a header whose declarations cross a call seam (task records, fragment types): its text
 // travels in the package and the linker puts it in front of the generated trampolines
@@ -190,6 +209,10 @@ inline int emit_main() {
                 empty_count, empty_by, init_owner)
 #define PL_EXPORT_TENSOR(name, result, dtype, rows, cols, home, layout, row_pitch)
 #define PL_IMPORT_TENSOR(name, fn, result, dtype, rows, cols, layout)
+#define PL_HOST_GROUP(params_group, provider_suffix)
+#define PL_HOST_ABI_TYPE(id, T)
+#define PL_HOST_SCALAR(id, name, kind)
+#define PL_HOST_CHANNEL(id, name, elem_bits, access, extents, optional)
 #define PL_FACT(name, value)
 #define PL_USES(handle)
 #define PL_PRELUDE(path)

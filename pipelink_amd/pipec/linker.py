@@ -101,6 +101,41 @@ def _math_flags(stages: list[Stage]) -> list[str]:
     return json.loads(next(iter(stamps)))
 
 
+def host_section(stages: list[Any], layout: dict[str, Any], arch: str) -> dict[str, Any] | None:
+    """link.json["host"]: the owner inventory a broker works from (the reference's host section,
+    link.py:1301 and host/broker.py:818-830) -- one group per stage that declared a params group:
+    its provider's entry points, the record types the provider must report, its caller-owned
+    channels and the scalars it reads; plus the stages whose params are plain blobs."""
+    groups, scalars, names = [], {}, set()
+    entries = {e["stage_id"]: e for e in layout["entries"]}
+    for stage in stages:
+        host = stage.manifest.get("host")
+        if not host:
+            continue
+        if host["params_group"] in names:
+            _fail("L-HOSTCHAN", f"stages.{stage.id}.host.params_group", "two stages declare the same params group",
+                  params_group=host["params_group"])
+        names.add(host["params_group"])
+        for sc in host["scalars"]:
+            known = scalars.setdefault(sc["id"], sc)
+            if known != sc:
+                _fail("L-HOSTCHAN", f"stages.{stage.id}.host.scalars.{sc['name']}", "owners disagree on a shared scalar",
+                      expected=known, actual=sc)
+        suffix = host["provider"]
+        groups.append({"params_group": host["params_group"], "owner": stage.id, "stage_ids": [stage.id],
+                       "params": {"bytes": entries[stage.id]["bytes"], "offset": entries[stage.id]["offset"]},
+                       "provider": {"symbols": {k: f"pipelink_params_{k}_{suffix}" for k in ("abi", "query", "build", "release")},
+                                    "abi_types": host["abi_types"]},
+                       "scalars": [sc["id"] for sc in host["scalars"]], "channels": host["channels"]})
+    if not groups:
+        return None
+    owned = {g["owner"] for g in groups}
+    return {"protocol": 2, "target": {"profile": arch}, "groups": groups,
+            "scalars": [scalars[k] for k in sorted(scalars)],
+            "params": {"blobs": [{"stage_id": e["stage_id"], "bytes": e["bytes"]} for e in layout["entries"]
+                                 if e["stage_id"] not in owned]}}
+
+
 def _to_bitcode(source: Path, out: Path, arch: str, flags: list[str], include_dirs: list[Path]) -> None:
     _run([HIPCC, f"--offload-arch={arch}", "-x", "hip", "-fgpu-rdc", "--cuda-device-only", "-emit-llvm", "-c", *flags,
           *[f"-I{d}" for d in [INCLUDE_DIR, *include_dirs]], source, "-o", out], f"compile.{source.name}")
@@ -176,7 +211,9 @@ def link(pipeline_path: str | Path, out_dir: str | Path, *, include_dirs: list[s
         if observed["vgpr_count"] > regs_cap:
             _fail("L-REGS", "observed.vgpr_count", "linked kernel needs more registers than the launch leaves per lane",
                   **observed)
+    host = host_section(stages, layout, arch)
     result = {
+        **({"host": host} if host else {}),
         "kernel_symbol": KERNEL_SYMBOL,
         "threads": solution.threads,
         "regs_cap": solution.regs_cap,

@@ -160,8 +160,21 @@ def assemble(registry: dict[str, Any], profile_name: str, source: Path) -> dict[
     if registry.get("tensor_exports") or registry.get("tensor_imports"):
         tensor = {"tensor": {"schema": "tensor-v1", "exports": registry.get("tensor_exports", []),
                              "imports": registry.get("tensor_imports", [])}}
+    host = {}
+    if registry.get("host_group"):
+        group = registry["host_group"][0]
+        channels = sorted(registry.get("host_channels", []), key=lambda c: c["id"])
+        if [c["id"] for c in channels] != list(range(1, len(channels) + 1)):
+            _fail("L-HOSTCHAN", "$.host.channels", "host channel ids must be 1..n without gaps", ids=[c["id"] for c in channels])
+        if params["bytes"] == 0:
+            _fail("L-HOSTCHAN", "$.host.params_group", "a stage without params cannot own a params group")
+        host = {"host": {"schema": "host-v2", "params_group": group["params_group"], "provider": group["provider"],
+                         "abi_types": sorted(registry.get("host_types", []), key=lambda t: t["id"]),
+                         "scalars": sorted(registry.get("host_scalars", []), key=lambda t: t["id"]),
+                         "channels": channels}}
     return {
         **tensor,
+        **host,
         "pipelink_abi": {"schema": "3.0", "target": {
             "profile": profile.name, "lto_arch": profile.lto_arch, "toolkit": TOOLKIT,
             "math": {"flags": DEVICE_FLAGS}}},

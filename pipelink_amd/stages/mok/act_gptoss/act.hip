@@ -171,6 +171,12 @@ PL_SERVE(act_init, "mok_act_init");
 PL_SERVE(act_fwd, "mok_act_fwd");
 // staging tile for the coalesced write-out; lives while no GEMM ring slot is in use
 PL_CLAIM("pipelink_mok_act_arena", "smem", 256 * 144 + 256 * 4, 1024, "phase:instr_act");
+// host contract (campaigns/mok/port/act/act.cu:280-330 in the reference)
+PL_HOST_GROUP("mok.act.params", "mok_act");
+PL_HOST_ABI_TYPE(2, MokActResidue);
+MOK_HOST_SCALARS();
+PL_HOST_CHANNEL(1, "hidden_q", 8, "write", "mok.routed_rows, mok.ld_q_i", false);
+PL_HOST_CHANNEL(2, "hidden_sc", 8, "write", "mok.routed_rows, mok.ld_sc_i", false);
 PL_USES("pipelink_mok_clamp");
 PL_USES("pipelink_mok_act_arena");
 PL_PRELUDE("../include/mok_abi.h");

@@ -137,6 +137,11 @@ PL_CALL(act_fwd, "mok_act_fwd",
 // schedule table: exclusive prefix sums of rows and row tiles for up to 256 experts
 PL_CLAIM("pipelink_mok_fw_sched", "smem", 2 * (256 + 1) * 4, 16, "kernel");
 PL_USES("pipelink_mok_fw_sched");
+// host contract: the schedule's owner
+PL_HOST_GROUP("mok.framework.params", "mok_framework");
+PL_HOST_ABI_TYPE(3, MokFrameworkParams);
+MOK_HOST_SCALARS();
+PL_HOST_CHANNEL(1, "tokens_per_expert", 32, "read", "mok.num_local_experts", false);
 PL_FACT("mok.framework.MAX_EXPERTS", 256);
 PL_PRELUDE("../include/mok_abi.h");
 PL_PRELUDE("../include/mok_device.hpp");

@@ -767,6 +767,24 @@ PL_CLAIM_RING("pipelink_mok_gemm_arena", "smem", -3 * 16384, "pipelink_mok_gemm_
 PL_USES("pipelink_mok_gemm_head");
 PL_USES("pipelink_mok_gemm_depth");
 PL_USES("pipelink_mok_gemm_arena");
+// host contract (the reference's PL_HOST_* block, campaigns/mok/port/gemm/gemm.cu:383-479): provider entry points
+// pipelink_params_*_mok_gemm, the records it reports, the caller's tensors
+PL_HOST_GROUP("mok.gemm.params", "mok_gemm");
+PL_HOST_ABI_TYPE(1, MokGemmResidue);
+PL_HOST_ABI_TYPE(4, MokMxView);
+MOK_HOST_SCALARS();
+PL_HOST_CHANNEL(1, "x_q", 8, "read", "mok.num_local_tokens, mok.ld_q_h", false);
+PL_HOST_CHANNEL(2, "x_sc", 8, "read", "mok.num_local_tokens, mok.ld_sc_h", false);
+PL_HOST_CHANNEL(3, "w_gate_q", 8, "read", "mok.num_local_experts, floor(mok.hidden,64), mok.intermediate, 64", false);
+PL_HOST_CHANNEL(4, "w_gate_sc", 8, "read", "mok.num_local_experts, ceil(mok.hidden,128), mok.intermediate, 4", false);
+PL_HOST_CHANNEL(5, "w_up_q", 8, "read", "mok.num_local_experts, floor(mok.hidden,64), mok.intermediate, 64", false);
+PL_HOST_CHANNEL(6, "w_up_sc", 8, "read", "mok.num_local_experts, ceil(mok.hidden,128), mok.intermediate, 4", false);
+PL_HOST_CHANNEL(7, "w_down_q", 8, "read", "mok.num_local_experts, floor(mok.intermediate,64), mok.hidden, 64", false);
+PL_HOST_CHANNEL(8, "w_down_sc", 8, "read", "mok.num_local_experts, ceil(mok.intermediate,128), mok.hidden, 4", false);
+PL_HOST_CHANNEL(9, "hidden_q", 8, "read", "mok.routed_rows, mok.ld_q_i", false);
+PL_HOST_CHANNEL(10, "hidden_sc", 8, "read", "mok.routed_rows, mok.ld_sc_i", false);
+PL_HOST_CHANNEL(11, "y", 16, "write", "mok.routed_rows, mok.hidden", false);
+PL_HOST_CHANNEL(12, "row_token", 32, "read", "mok.routed_rows", true);  // left out: routed rows are tokens
 PL_FACT("mok.gemm.TILE_X", 256);
 PL_FACT("mok.gemm.TILE_W", 256);
 PL_FACT("mok.gemm.K_SLOT", 64);

@@ -100,6 +100,22 @@ typedef struct MokFrameworkParams {
   int32_t reserved;
 } MokFrameworkParams;
 
+/* The shared scalars every owner of this pipeline is handed (ids of include/plk_host_abi_v2.h); a stage source
+ * invokes this among its annotations, after <pipelink/stage.hpp>. */
+#define MOK_HOST_SCALARS()                                \
+  PL_HOST_SCALAR(1, "mok.num_local_tokens", "i64");       \
+  PL_HOST_SCALAR(2, "mok.hidden", "i64");                 \
+  PL_HOST_SCALAR(3, "mok.intermediate", "i64");           \
+  PL_HOST_SCALAR(4, "mok.num_local_experts", "i64");      \
+  PL_HOST_SCALAR(10, "mok.swiglu_limit", "f64");          \
+  PL_HOST_SCALAR(11, "mok.pass", "i64");                  \
+  PL_HOST_SCALAR(12, "mok.precision", "i64");             \
+  PL_HOST_SCALAR(60, "mok.routed_rows", "i64");           \
+  PL_HOST_SCALAR(61, "mok.ld_q_h", "i64");                \
+  PL_HOST_SCALAR(62, "mok.ld_q_i", "i64");                \
+  PL_HOST_SCALAR(63, "mok.ld_sc_h", "i64");               \
+  PL_HOST_SCALAR(64, "mok.ld_sc_i", "i64")
+
 /* First argument of every owner export (pack/include/pipelink/host_view.h in the reference). */
 #ifndef PIPELINK_HOST_VIEW_DEFINED
 #define PIPELINK_HOST_VIEW_DEFINED

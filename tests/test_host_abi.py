@@ -19,16 +19,19 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SCALARS = {"mok.num_local_tokens": 512, "mok.hidden": 320, "mok.intermediate": 192, "mok.num_local_experts": 4,
            "mok.swiglu_limit": 7.0, "mok.pass": 1, "mok.precision": 1, "mok.routed_rows": 1024, "mok.ld_q_h": 384,
            "mok.ld_q_i": 256, "mok.ld_sc_h": 16, "mok.ld_sc_i": 16}
-LINK = {"threads": 256, "dyn_smem_bytes": 161800, "kernel_symbol": "pipelink_kernel", "workgroups_per_cu": 1,
+# the owner inventory is what the built pipeline's link recorded from the stages' PL_HOST_* declarations
+HOST = json.loads(open(os.path.join(ROOT, "pipelink_amd", "stages", "mok", "build", "link", "link.json")).read())["host"]
+LINK = {"threads": 256, "dyn_smem_bytes": 161800, "kernel_symbol": "pipelink_kernel", "workgroups_per_cu": 1, "host": HOST,
         "params": {"total_bytes": 344, "entries": [{"stage_id": "mok.framework", "offset": 0, "bytes": 40},
                                                    {"stage_id": "mok.gemm", "offset": 40, "bytes": 264},
                                                    {"stage_id": "mok.act", "offset": 304, "bytes": 40}]}}
+GROUPS = {g["owner"]: g for g in HOST["groups"]}
 
 
 def _resources(scalars=SCALARS, row_token=True):
     """Fake device addresses (nothing is dereferenced on the host): 1 MiB apart, 256-byte aligned."""
     out, addr = {}, 0x7F0000000000
-    for stage, chans in broker._shapes(scalars).items():
+    for stage, chans in broker.channel_shapes(LINK, scalars).items():
         out[stage] = {}
         for name, (bits, _, extents) in chans.items():
             if name == "row_token" and not row_token:
@@ -43,15 +46,16 @@ def _resources(scalars=SCALARS, row_token=True):
 
 def test_abi_report_matches_the_ctypes_mirrors():
     lib = load_library()
-    for stage in broker.OWNERS:
-        rep = broker.Owner(lib, stage).report()          # raises on any size / alignment / digest mismatch
-        assert rep.entry_count == 20 + len(broker.OWNERS[stage][1])
+    assert set(GROUPS) == {"mok.framework", "mok.gemm", "mok.act"}
+    for stage, group in GROUPS.items():
+        rep = broker.Owner(lib, group).report()          # raises on any size / alignment / digest mismatch
+        assert rep.entry_count == 20 + len(group["provider"]["abi_types"])
     assert sizeof(broker.MokGemmResidue) == 264 and sizeof(broker.MokActResidue) == 40 and sizeof(broker.MokFrameworkParams) == 40
 
 
 def test_abi_report_rejects_wrong_version_capacity_and_ids():
     lib = load_library()
-    owner = broker.Owner(lib, "mok.gemm")
+    owner = broker.Owner(lib, GROUPS["mok.gemm"])
     rep = broker.AbiReport()
     rep.header = broker.Header(3, sizeof(rep))
     assert owner.abi(byref(rep)) == 1                     # PLK_E_VERSION
@@ -117,8 +121,8 @@ def test_provider_and_broker_reject_bad_inputs(mutate, status):
 def test_build_checks_the_resource_records_itself():
     """Call build directly with a resource smaller than the demand: PLK_E_RESOURCE, and no session."""
     lib = load_library()
-    owner = broker.Owner(lib, "mok.act")
-    shared = broker._Scalars(SCALARS)
+    owner = broker.Owner(lib, GROUPS["mok.act"])
+    shared = broker._Scalars(SCALARS, HOST["scalars"])
     common = broker.Common()
     common.header = broker.Header(2, sizeof(common))
     common.channel_count, common.shared = 2, shared.pointer
@@ -135,3 +139,36 @@ def test_build_checks_the_resource_records_itself():
     assert owner.build(byref(common), None, byref(r), out, 40, None, 1, byref(session)) == 2      # transfers are not reported
     assert owner.build(byref(common), ctypes.c_void_p(1), byref(r), out, 40, None, 0, byref(session)) == 3   # args must be null
     assert owner.release(ctypes.c_void_p(1)) == 7 and owner.release(None) == 0
+
+
+def test_owner_inventory_comes_from_the_link():
+    """What the stages declared with PL_HOST_* is what the link recorded and the broker works from."""
+    assert HOST["protocol"] == 2 and HOST["params"]["blobs"] == []
+    gemm = GROUPS["mok.gemm"]
+    assert gemm["params_group"] == "mok.gemm.params" and gemm["provider"]["symbols"]["build"] == "pipelink_params_build_mok_gemm"
+    assert [c["name"] for c in gemm["channels"]] == ["x_q", "x_sc", "w_gate_q", "w_gate_sc", "w_up_q", "w_up_sc", "w_down_q",
+                                                     "w_down_sc", "hidden_q", "hidden_sc", "y", "row_token"]
+    assert [c["name"] for c in gemm["channels"] if c["optional"]] == ["row_token"]
+    assert {t["name"]: t["bytes"] for t in gemm["provider"]["abi_types"]} == {"MokGemmResidue": 264, "MokMxView": 48}
+    assert [s["id"] for s in HOST["scalars"]] == [1, 2, 3, 4, 10, 11, 12, 60, 61, 62, 63, 64]
+    assert broker.evaluate_extents("mok.num_local_experts, floor(mok.hidden,64), ceil(mok.intermediate, 128), 4", SCALARS) == (4, 5, 2, 4)
+    with pytest.raises(PlkError):
+        broker.evaluate_extents("mok.hidden * 2", SCALARS)
+
+
+def test_broker_refuses_a_link_without_inventory_or_with_foreign_records():
+    res = _resources()
+    bare = {k: v for k, v in LINK.items() if k != "host"}
+    with pytest.raises(PlkError) as err:
+        broker.plan(bare, res, SCALARS, compute_units=256)
+    assert err.value.status == 4 and "host section" in str(err.value)
+    other = json.loads(json.dumps(LINK))
+    other["host"]["groups"][0]["provider"]["abi_types"][0]["bytes"] += 8       # a record this broker mirrors differently
+    with pytest.raises(PlkError) as err:
+        broker.plan(other, res, SCALARS, compute_units=256)
+    assert err.value.status == 1
+    gone = json.loads(json.dumps(LINK))
+    gone["host"]["groups"][1]["provider"]["symbols"]["query"] = "pipelink_params_query_nobody"
+    with pytest.raises(PlkError) as err:
+        broker.plan(gone, res, SCALARS, compute_units=256)
+    assert err.value.status == 4 and "missing provider export" in str(err.value)

@@ -166,6 +166,10 @@ class MemoryBackend:
 def test_hostless_launcher_params_contract(cell):
     link = json.loads((cell[0] / "link" / "link.json").read_text())
     image = cell[0] / "link" / "pipeline.hsaco"
+    with pytest.raises(LaunchError) as err:      # a link whose stages declared owners is opened through its providers
+        open_hostless(link, buffers={}, params=lambda a: {}, grid=(1,), backend=MemoryBackend(), image=image)
+    assert err.value.failures[0].path == "launch.host"
+    assert [g["owner"] for g in link.pop("host")["groups"]] == ["mok.framework", "mok.gemm", "mok.act"]
     be = MemoryBackend()
     seen = {}
 
