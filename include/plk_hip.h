@@ -63,6 +63,14 @@ int plk_hip_synchronize(void* stream);                               /* CudaBack
 
 int plk_hip_stream_create(void** stream);
 int plk_hip_stream_destroy(void* stream);
+/* Graph capture of one stream (CudaBackend.capture, host/cuda.py:267-286; Graph.launch / close, :358-382).  The stream
+ * must be one made by plk_hip_stream_create.  While a stream is captured plk_hip_zero / plk_hip_fill_u8 record a
+ * fill kernel, not a memset node; uploads and readbacks synchronise and cannot be captured. */
+int plk_hip_graph_begin(void* stream);
+int plk_hip_graph_end(void* stream, void** graph, void** executable);   /* ends the capture and instantiates it */
+int plk_hip_graph_abort(void* stream);                                  /* ends a capture whose body failed; keeps nothing */
+int plk_hip_graph_launch(void* executable, void* stream);
+int plk_hip_graph_destroy(void* graph, void* executable);
 int plk_hip_event_create(void** event);                              /* CudaBackend.event_create */
 int plk_hip_event_record(void* event, void* stream);
 int plk_hip_event_synchronize(void* event);

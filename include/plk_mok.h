@@ -66,7 +66,10 @@ typedef struct plk_mok_session plk_mok_session;
 
 int plk_mok_session_create(const void* image, size_t image_bytes, const plk_mok_link_info* link, plk_mok_session** out);
 int plk_mok_session_destroy(plk_mok_session* s);
-/* both passes; or one of them (pass 1 = gate/up + SwiGLU + requant, pass 2 = down) */
+/* both passes; or one of them (pass 1 = gate/up + SwiGLU + requant, pass 2 = down).  The session keeps the params image
+ * of the last problem per pass on the device: a call with the same problem only launches (and can be captured into a
+ * graph); a call with another problem first uploads its image, which synchronises the stream -- on a stream that is
+ * being captured that call returns PLK_E_CONTRACT. */
 int plk_mok_forward(plk_mok_session* s, const plk_mok_problem* p, void* stream);
 int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass, void* stream);
 

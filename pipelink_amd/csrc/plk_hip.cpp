@@ -33,6 +33,12 @@ int fail_msg(int code, const char* what) {
 }
 }  // namespace
 
+// Fill for a stream that is being captured into a graph: a memset node recorded there is not replayed
+// reliably on this stack, a kernel node is.
+__global__ void plk_fill_kernel(unsigned char* dst, unsigned char value, size_t bytes) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < bytes; i += (size_t)gridDim.x * blockDim.x) dst[i] = value;
+}
+
 #define PLK_HIP_TRY(code, expr)                        \
   do {                                                 \
     hipError_t e_ = (expr);                            \
@@ -93,7 +99,56 @@ int plk_hip_zero(uint64_t addr, size_t bytes, void* stream) { return plk_hip_fil
 
 int plk_hip_fill_u8(uint64_t addr, int value, size_t bytes, void* stream) {
   if (!bytes) return PLK_OK;
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (stream) PLK_HIP_TRY(PLK_E_RESOURCE, hipStreamIsCapturing((hipStream_t)stream, &capturing));
+  if (capturing == hipStreamCaptureStatusActive) {
+    const unsigned blocks = (unsigned)((bytes + 256 * 64 - 1) / (256 * 64) < 4096 ? (bytes + 256 * 64 - 1) / (256 * 64) : 4096);
+    hipLaunchKernelGGL(plk_fill_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (unsigned char*)(uintptr_t)addr,
+                       (unsigned char)value, bytes);
+    PLK_HIP_TRY(PLK_E_RESOURCE, hipGetLastError());
+    return PLK_OK;
+  }
   PLK_HIP_TRY(PLK_E_RESOURCE, hipMemsetAsync((void*)(uintptr_t)addr, value, bytes, (hipStream_t)stream));
+  return PLK_OK;
+}
+
+int plk_hip_graph_begin(void* stream) {
+  if (!stream) return fail_msg(PLK_E_ARGUMENT, "plk_hip_graph_begin: the default stream cannot be captured; create one");
+  PLK_HIP_TRY(PLK_E_RESOURCE, hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+  return PLK_OK;
+}
+
+int plk_hip_graph_end(void* stream, void** graph, void** executable) {
+  if (!graph || !executable) return fail_msg(PLK_E_ARGUMENT, "plk_hip_graph_end: null output");
+  hipGraph_t g = nullptr;
+  PLK_HIP_TRY(PLK_E_RESOURCE, hipStreamEndCapture((hipStream_t)stream, &g));
+  hipGraphExec_t e = nullptr;
+  const hipError_t err = hipGraphInstantiate(&e, g, nullptr, nullptr, 0);
+  if (err != hipSuccess) {
+    (void)hipGraphDestroy(g);
+    return fail(PLK_E_RESOURCE, "hipGraphInstantiate", err);
+  }
+  *graph = (void*)g;
+  *executable = (void*)e;
+  return PLK_OK;
+}
+
+int plk_hip_graph_abort(void* stream) {
+  hipGraph_t g = nullptr;
+  const hipError_t err = hipStreamEndCapture((hipStream_t)stream, &g);
+  if (g) (void)hipGraphDestroy(g);
+  if (err != hipSuccess && err != hipErrorStreamCaptureInvalidated) return fail(PLK_E_RELEASE, "hipStreamEndCapture", err);
+  return PLK_OK;
+}
+
+int plk_hip_graph_launch(void* executable, void* stream) {
+  PLK_HIP_TRY(PLK_E_RESOURCE, hipGraphLaunch((hipGraphExec_t)executable, (hipStream_t)stream));
+  return PLK_OK;
+}
+
+int plk_hip_graph_destroy(void* graph, void* executable) {
+  if (executable) PLK_HIP_TRY(PLK_E_RELEASE, hipGraphExecDestroy((hipGraphExec_t)executable));
+  if (graph) PLK_HIP_TRY(PLK_E_RELEASE, hipGraphDestroy((hipGraph_t)graph));
   return PLK_OK;
 }
 

@@ -126,6 +126,11 @@ int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass,
   std::memcpy(image.data() + s->link.gemm_offset, &g, sizeof g);
   std::memcpy(image.data() + s->link.act_offset, &a, sizeof a);
   if (image != s->params_host[slot]) {
+    // a new problem: its params image goes to the device first, which synchronises and cannot be part of a graph
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (stream && hipStreamIsCapturing((hipStream_t)stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusActive)
+      return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_forward: this problem's params image is not on the device yet; run the "
+                                               "forward once before capturing it into a graph");
     rc = plk_hip_upload(s->params_dev[slot], image.data(), image.size(), stream);
     if (rc != PLK_OK) return rc;
     s->params_host[slot].swap(image);

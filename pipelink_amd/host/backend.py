@@ -58,6 +58,11 @@ SIGNATURES = {
     "plk_hip_synchronize": (c_int, [c_void_p]),
     "plk_hip_stream_create": (c_int, [POINTER(c_void_p)]),
     "plk_hip_stream_destroy": (c_int, [c_void_p]),
+    "plk_hip_graph_begin": (c_int, [c_void_p]),
+    "plk_hip_graph_end": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p)]),
+    "plk_hip_graph_abort": (c_int, [c_void_p]),
+    "plk_hip_graph_launch": (c_int, [c_void_p, c_void_p]),
+    "plk_hip_graph_destroy": (c_int, [c_void_p, c_void_p]),
     "plk_hip_event_create": (c_int, [POINTER(c_void_p)]),
     "plk_hip_event_record": (c_int, [c_void_p, c_void_p]),
     "plk_hip_event_synchronize": (c_int, [c_void_p]),
@@ -102,20 +107,93 @@ def check(lib, status: int) -> None:
         raise PlkError(status, (lib.plk_hip_last_error() or b"").decode("utf-8", "replace"))
 
 
+class _Current:
+    """What HipBackend.current() returns: the device is already current; usable as ``with backend.current():``."""
+
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+class Graph:
+    """An instantiated graph replaying exactly the work captured on one stream (host/cuda.py:358-388 in the reference)."""
+
+    def __init__(self, backend: "HipBackend", graph: int, executable: int):
+        self._backend, self._graph, self.executable, self.closed = backend, graph, executable, False
+
+    def launch(self, stream: int | None = None) -> None:
+        check(self._backend.lib, self._backend.lib.plk_hip_graph_launch(self.executable, self._backend._s(stream)))
+
+    def close(self) -> None:
+        if self.closed:
+            return
+        self.closed = True
+        self._backend._graphs.remove(self)
+        if not self._backend.lost:
+            check(self._backend.lib, self._backend.lib.plk_hip_graph_destroy(self._graph, self.executable))
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+
 class HipBackend:
-    """Device memory, events and launches on one GPU; ``stream`` is a raw ``hipStream_t`` (0 = default)."""
+    """Device memory, events, launches and graph capture on one GPU; ``stream`` is a raw ``hipStream_t`` (0 = default).
+
+    The method set is the reference's ``CudaBackend`` (host/cuda.py:118-356): allocate / free / zero / upload /
+    readback / synchronize / event_* / launch / capture / current / abandon / close, ``stream_token``,
+    ``observations``."""
 
     def __init__(self, device: int = 0, stream: int = 0):
         self.lib = load_library()
         self.device = device
         self.stream_token = stream
+        self.lost = self.closed = False
         check(self.lib, self.lib.plk_hip_set_device(device))
-        self.observations: dict = {}
         self._allocations: set[int] = set()
+        self._graphs: list[Graph] = []
+        self._streams: list[int] = []
+        info = self.info()
+        self.observations: dict = {"device_ordinal": device, "arch": info.arch.decode().split(":")[0],
+                                   "observed_cu_count": info.compute_units, "wavefront_size": info.wavefront_size,
+                                   "max_lds_per_workgroup": info.max_lds_per_workgroup,
+                                   "max_threads": info.max_threads_per_workgroup, "l2_bytes": info.l2_bytes,
+                                   "total_memory": info.total_memory}
 
-    # -- CudaBackend.current()
-    def current(self) -> None:
+    # -- CudaBackend.current(): one device, one context -- making it current is setting the device
+    def current(self) -> _Current:
         check(self.lib, self.lib.plk_hip_set_device(self.device))
+        return _Current()
+
+    def stream_create(self) -> int:
+        """A stream of default priority that close() destroys (graph capture needs one: stream 0 cannot be captured)."""
+        s = c_void_p()
+        check(self.lib, self.lib.plk_hip_stream_create(byref(s)))
+        self._streams.append(s.value)
+        return s.value
+
+    def capture(self, stream: int, body) -> Graph:
+        """Record what ``body()`` enqueues on ``stream`` and instantiate it.  Fills issued in the body are recorded as
+        kernels; an upload or a readback in the body fails the capture."""
+        check(self.lib, self.lib.plk_hip_graph_begin(c_void_p(stream)))
+        try:
+            body()
+        except BaseException:
+            self.lib.plk_hip_graph_abort(c_void_p(stream))
+            raise
+        graph, executable = c_void_p(), c_void_p()
+        check(self.lib, self.lib.plk_hip_graph_end(c_void_p(stream), byref(graph), byref(executable)))
+        result = Graph(self, graph.value, executable.value)
+        self._graphs.append(result)
+        return result
+
+    def abandon(self) -> None:
+        """After a failed synchronisation: nothing this backend allocated is reused or freed."""
+        self.lost = True
 
     def info(self) -> DeviceInfo:
         out = DeviceInfo()
@@ -192,9 +270,24 @@ class HipBackend:
         check(self.lib, self.lib.plk_hip_launch(function, byref(g), byref(b), dyn_lds_bytes, self._s(stream), params_addr))
 
     def close(self) -> None:
-        for addr in sorted(self._allocations):
-            self.lib.plk_hip_free(addr)
+        if self.closed:
+            return
+        self.closed = True
+        for graph in list(self._graphs):
+            graph.close()
+        if not self.lost:
+            for addr in sorted(self._allocations):
+                self.lib.plk_hip_free(addr)
+            for stream in self._streams:
+                self.lib.plk_hip_stream_destroy(c_void_p(stream))
         self._allocations.clear()
+        self._streams.clear()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
 
     def _s(self, stream):
         return c_void_p(self.stream_token if stream is None else stream)

@@ -23,6 +23,7 @@ from ctypes import (POINTER, Structure, byref, c_int64, c_size_t, c_uint8, c_uin
 from dataclasses import dataclass
 from typing import Any, Mapping
 
+from .fixture import Domain, Fixture, Resource  # noqa: F401  (the reference exposes them beside open_host)
 from .backend import PlkError, load_library
 
 ABI_V2 = 2
@@ -216,14 +217,6 @@ def layout_digest(name: str, mirror: type[Structure]) -> bytes:
     """SHA-256 of "type{member@offset+size;...}" -- what a provider reports as compiler_layout."""
     text = name + "{" + "".join(f"{m}@{getattr(mirror, m).offset}+{getattr(mirror, m).size};" for m, *_ in mirror._fields_) + "}"
     return hashlib.sha256(text.encode()).digest()
-
-
-@dataclass
-class Resource:
-    """One caller-owned device allocation (host/fixture.py:22-40 in the reference)."""
-    address: int
-    allocation_bytes: int
-    origin_byte_offset: int = 0
 
 
 def _header(record: Structure) -> None:

@@ -242,6 +242,55 @@ def test_broker_route_gives_the_same_bytes_as_the_forward_entry(cell):
     assert torch.equal(t["y"].cpu().view(torch.int16), want[2].view(torch.int16))
 
 
+def test_forward_captured_in_a_graph_replays_to_the_same_bytes(cell):
+    """HipBackend.capture / Graph.launch (the reference's CudaBackend.capture, host/cuda.py:267-286): the forward's
+    two launches and a fill recorded on a created stream, replayed three times with eager work and
+    synchronisations in between, every replay against the eager result."""
+    from pipelink_amd.host import mok_inputs
+    from pipelink_amd.host.backend import HipBackend, PlkError
+    from pipelink_amd.host.mok import scale_pitch, weight_codes_to_k64_tiled, weight_scales_to_slot_major
+
+    T, H, I, E, k = 300, 320, 192, 4, 2
+    inp = mok_inputs.generate(T, H, I, E, k, seed=5)
+    want = _run(cell[0], inp, H, I)
+    dev = torch.device("cuda:0")
+    d = {n: v.to(dev) for n, v in inp.__dict__.items()}
+    for name, kk in (("w_gate", H), ("w_up", H), ("w_down", I)):
+        d[name + "_sc"] = weight_scales_to_slot_major(d[name + "_sc"], kk)
+        d[name + "_q"] = weight_codes_to_k64_tiled(d[name + "_q"], kk)
+    rows = int(inp.tokens_per_expert.sum())
+    hq = torch.zeros((rows, I), dtype=torch.uint8, device=dev)
+    hsc = torch.zeros((rows, scale_pitch(I)), dtype=torch.uint8, device=dev)
+    y = torch.zeros((rows, H), dtype=torch.bfloat16, device=dev)
+    prob = cell[0].problem(hidden_q=hq, hidden_sc=hsc, y=y, swiglu_limit=7.0, **d)
+    torch.cuda.synchronize()
+    with HipBackend(0) as be:
+        stream = be.stream_create()
+        with pytest.raises(PlkError):                       # the default stream cannot be captured
+            be.capture(0, lambda: None)
+        with pytest.raises(ZeroDivisionError):              # a body that fails ends the capture and keeps nothing
+            be.capture(stream, lambda: 1 // 0)
+
+        def body():
+            be.fill(hq.data_ptr(), 0xFF, hq.numel(), stream)      # recorded as a fill kernel
+            cell[0].forward(prob, stream=stream)
+        with pytest.raises(PlkError) as err:                # a problem the session has not seen needs an upload first
+            be.capture(stream, body)
+        assert err.value.status == 4 and "once before capturing" in str(err.value)
+        cell[0].forward(prob, stream=stream)                # now its params image is on the device
+        be.synchronize(stream)
+        with be.capture(stream, body) as graph:
+            for replay in range(3):
+                y.fill_(float("nan"))                        # eager work between the replays
+                hsc.fill_(0xFF)
+                torch.cuda.synchronize()
+                graph.launch(stream)
+                be.synchronize(stream)
+                assert np.array_equal(hq.cpu().numpy(), want[0]) and np.array_equal(hsc.cpu().numpy(), want[1]), replay
+                assert torch.equal(y.cpu().view(torch.int16), want[2].view(torch.int16)), replay
+        assert be.observations["arch"].startswith("gfx") and be.observations["observed_cu_count"] > 0
+
+
 def test_argument_errors_are_reported_not_launched(cell):
     from pipelink_amd.host import mok_inputs
     from pipelink_amd.host.backend import PlkError

@@ -172,3 +172,44 @@ def test_broker_refuses_a_link_without_inventory_or_with_foreign_records():
     with pytest.raises(PlkError) as err:
         broker.plan(gone, res, SCALARS, compute_units=256)
     assert err.value.status == 4 and "missing provider export" in str(err.value)
+
+
+def test_fixture_owns_buffers_until_it_closes():
+    """pipec2.host.fixture.Fixture's contract (fixture.py:44-96 in the reference) on a host-memory backend."""
+    from pipelink_amd.host.fixture import Domain, Fixture
+
+    class Memory:
+        lost = False
+
+        def __init__(self):
+            self.mem, self.next, self.freed, self.synced = {}, 0x1000, [], 0
+
+        def allocate(self, size, align=256):
+            addr, self.next = self.next, self.next + (size + 255) // 256 * 256
+            self.mem[addr] = bytearray(size)
+            return addr
+
+        def free(self, addr): self.freed.append(addr)
+        def upload(self, addr, data, stream=None): self.mem[addr][:len(data)] = data
+        def zero(self, addr, size, stream=None): self.mem[addr][:size] = bytes(size)
+        def readback(self, addr, size, stream=None): return bytes(self.mem[addr][:size])
+        def synchronize(self, stream=None): self.synced += 1
+
+    be = Memory()
+    with Fixture(be) as fx:
+        a = fx.tensor("a", data=b"\x01\x02\x03\x04", allocation_bytes=4)
+        out = fx.tensor("out", data=None, allocation_bytes=8, output=True)
+        assert (a.address, a.allocation_bytes) == (0x1000, 4) and out.address == 0x1100
+        with pytest.raises(ValueError):
+            fx.tensor("a", data=None, allocation_bytes=4)              # a name is lent once
+        with pytest.raises(ValueError):
+            fx.tensor("b", data=b"\x00", allocation_bytes=4)           # data must cover the allocation
+        be.mem[out.address][:] = b"ABCDEFGH"
+        assert fx.readback() == {"out": b"ABCDEFGH"}
+    assert be.freed == [0x1100, 0x1000] and be.synced == 1            # reverse order, after a drain
+    lost = Memory()
+    lost.lost = True
+    with Fixture(lost) as fx:
+        fx.tensor("a", data=None, allocation_bytes=4)
+    assert lost.freed == []                                           # an abandoned backend's memory is not reused
+    assert Domain(0, 1).world == 1
