@@ -337,13 +337,19 @@ class HostSession:
 
 
 def plan(link: Mapping[str, Any], resources: Mapping[str, Mapping[str, Resource]], scalars: Mapping[str, Any], *,
-         compute_units: int, lib: ctypes.CDLL | None = None, stream_token: int = 0) -> tuple[bytes, dict[str, Any], list[Owner]]:
+         compute_units: int, lib: ctypes.CDLL | None = None, stream_token: int = 0,
+         providers: Mapping[str, ctypes.CDLL] | None = None) -> tuple[bytes, dict[str, Any], list[Owner]]:
     """report -> query -> build for every owner; returns (params image, launch geometry, owners).
 
     Host-only: touches no device memory.  ``resources`` maps stage id -> channel name -> Resource."""
-    lib = lib or load_library()
     host = host_inventory(link)
     groups = {g["owner"]: g for g in host["groups"]}
+    if providers is not None:  # one library per params group, as the reference's open_host takes them (broker.py:824-827)
+        if set(providers) != {g["params_group"] for g in host["groups"]}:
+            raise PlkError(4, "providers must exactly resolve the link's params groups: "
+                              f"expected {sorted(g['params_group'] for g in host['groups'])}, got {sorted(providers)}")
+    else:
+        lib = lib or load_library()
     entries = {e["stage_id"]: e for e in link["params"]["entries"]}
     blobs = {b["stage_id"] for b in host["params"]["blobs"] if b["bytes"]}
     if set(entries) - blobs != set(groups) or set(resources) != set(groups):
@@ -361,7 +367,7 @@ def plan(link: Mapping[str, Any], resources: Mapping[str, Mapping[str, Resource]
     keep: list[Any] = [shared]
     try:
         for stage_id in (s["stage_id"] for s in link["params"]["entries"] if s["stage_id"] in groups):
-            owner = Owner(lib, groups[stage_id])
+            owner = Owner(providers[groups[stage_id]["params_group"]] if providers is not None else lib, groups[stage_id])
             owners.append(owner)
             rep = owner.report()
             names = list(shapes[stage_id])
@@ -432,7 +438,7 @@ def plan(link: Mapping[str, Any], resources: Mapping[str, Mapping[str, Resource]
 
 
 def open_host(link: Mapping[str, Any], image: bytes, resources: Mapping[str, Mapping[str, Resource]],
-              scalars: Mapping[str, Any], backend: Any) -> HostSession:
+              scalars: Mapping[str, Any], backend: Any, providers: Mapping[str, ctypes.CDLL] | None = None) -> HostSession:
     """Load the code object, plan the params image through the providers, put it on the device."""
     session = HostSession(backend)
     session.module = backend.module_load(image)
@@ -440,7 +446,7 @@ def open_host(link: Mapping[str, Any], image: bytes, resources: Mapping[str, Map
         session.function = backend.module_function(session.module, link["kernel_symbol"], link["dyn_smem_bytes"])
         session.image, session.geometry, session.owners = plan(link, resources, scalars,
                                                                compute_units=backend.info().compute_units,
-                                                               stream_token=backend.stream_token)
+                                                               stream_token=backend.stream_token, providers=providers)
         session.params_addr = backend.allocate(len(session.image), 256)
         backend.upload(session.params_addr, session.image)
         backend.synchronize()

@@ -6,7 +6,9 @@ its contents are read back stays on this side of the C seam: a ``Fixture`` owns 
 its backend until the host session that borrowed them has closed."""
 from __future__ import annotations
 
+import json
 from dataclasses import dataclass
+from pathlib import Path
 from typing import Any, NamedTuple
 
 
@@ -72,3 +74,30 @@ class Fixture:
             for address in reversed(self._allocations):
                 self.backend.free(address)
         self._allocations.clear()
+
+
+def load_inputs(path: str | Path, fixture: Fixture) -> tuple[dict[str, Any], dict[str, Path]]:
+    """Caller scalars and buffers for ``pipec launch --host-inputs`` (the reference's ``load_inputs``,
+    host/fixture.py:122-156): ``{"scalars": {...}, "resources": {name: {"data": FILE | null, "allocation_bytes": n,
+    ["alignment": a,] ["origin_byte_offset": o,] ["output": FILE]}}}``, paths relative to the JSON.  A resource
+    without data is zeroed; one that names an output file is read back after the launch.  The tensor metadata the
+    reference's records carry besides (extents, strides, dtype) is accepted and not needed: the link states every
+    channel's extents.  Returns (scalars, {name: output path})."""
+    path = Path(path)
+    obj = json.loads(path.read_text())
+    if not isinstance(obj, dict) or set(obj) != {"scalars", "resources"}:
+        raise ValueError("host inputs require exactly scalars and resources objects")
+    if not isinstance(obj["scalars"], dict) or not isinstance(obj["resources"], dict):
+        raise ValueError("host scalars/resources must be objects")
+    known = {"data", "allocation_bytes", "extents", "bit_strides", "dtype_id", "alignment", "origin_byte_offset",
+             "origin_bit_offset", "output"}
+    outputs: dict[str, Path] = {}
+    for name, item in obj["resources"].items():
+        if not isinstance(item, dict) or not {"data", "allocation_bytes"} <= set(item) or set(item) - known:
+            raise ValueError(f"invalid fixture declaration for {name}")
+        data = None if item["data"] is None else (path.parent / item["data"]).read_bytes()
+        fixture.tensor(name, data=data, allocation_bytes=item["allocation_bytes"], alignment=item.get("alignment", 256),
+                       origin_byte_offset=item.get("origin_byte_offset", 0), output=item.get("output") is not None)
+        if item.get("output") is not None:
+            outputs[name] = path.parent / item["output"]
+    return obj["scalars"], outputs

@@ -34,7 +34,8 @@ def main(argv: list[str] | None = None) -> int:
     p.add_argument("--params", metavar="PY_FILE:FUNCTION", help="Python builder: device addresses -> stage params bytes")
     p.add_argument("--blob", action="append", default=[], metavar="STAGE_ID=PATH", help="already-built stage params blob")
     p.add_argument("--output", action="append", default=[], metavar="NAME=FILE.npy", help="save a buffer after the launch")
-    p.add_argument("--provider", action="append", default=[], metavar="GROUP=SO", help="(host links are opened through the broker)")
+    p.add_argument("--provider", action="append", default=[], metavar="GROUP=SO", help="owner provider shared object keyed by params group")
+    p.add_argument("--host-inputs", help="caller scalar and buffer JSON for a link with a host section")
     p.add_argument("--device", type=int, default=0)
     p = sub.add_parser("clauses", help="list the named diagnostics")
     p.add_argument("--json", action="store_true")
@@ -63,7 +64,7 @@ def main(argv: list[str] | None = None) -> int:
             grid = tuple(int(v) for v in args.grid.split(",")) if args.grid else None
             print(json.dumps(launcher.launch(args.link_json, grid=grid, buffers=pairs(args.buffer), params=args.params,
                                              blobs=pairs(args.blob), outputs=pairs(args.output), providers=pairs(args.provider),
-                                             device=args.device), indent=1))
+                                             host_inputs=args.host_inputs, device=args.device), indent=1))
         elif args.cmd == "clauses":
             rows = [{"id": c, "phase": CLAUSE_PHASES[c], "description": CLAUSES[c]} for c in sorted(CLAUSES)]
             print(json.dumps(rows, indent=1) if args.json else "\n".join(f"{r['id']:12s} {r['phase']:9s} {r['description']}" for r in rows))

@@ -171,13 +171,16 @@ def _load_params_function(spec: str) -> Callable[[dict[str, int]], dict[str, byt
 
 def launch(link_json: str | Path, *, grid: tuple[int, ...] | None, buffers: dict[str, str] | None = None,
            params: str | None = None, blobs: dict[str, str | Path] | None = None, outputs: dict[str, str | Path] | None = None,
-           providers: dict[str, str] | None = None, device: int = 0, backend=None) -> dict[str, Any]:
-    """One launch on the host-less route, as ``pipec launch`` runs it (pipec/src/pipec2/launcher.py:284-333
-    in the reference): buffers from ``NAME -> FILE.npy | SHAPE:DTYPE``, params either from a Python
+           providers: dict[str, str] | None = None, host_inputs: str | Path | None = None, device: int = 0,
+           backend=None) -> dict[str, Any]:
+    """One launch, as ``pipec launch`` runs it (pipec/src/pipec2/launcher.py:284-333 in the reference).  A link with
+    a host section goes through its providers (``providers`` = params group -> shared library, ``host_inputs`` = the
+    caller's scalars and buffers, see ``host.fixture.load_inputs``).  Any other link takes the host-less route: buffers from ``NAME -> FILE.npy | SHAPE:DTYPE``, params either from a Python
     builder ``PY_FILE:FUNCTION`` (device addresses -> stage bytes) or from ready-made blobs
     ``STAGE_ID -> file``; named buffers are saved as .npy afterwards.  Returns the report the CLI prints."""
-    if providers:
-        _fail("L-LAUNCH", "launch.providers", "links with host providers are opened through the host broker, not this route")
+    link_obj = json.loads(Path(link_json).read_text())
+    if link_obj.get("host") or providers or host_inputs:
+        return _launch_host(Path(link_json), link_obj, providers or {}, host_inputs, device, backend, grid, buffers, params, blobs)
     if grid is None:
         _fail("L-LAUNCH", "launch.grid", "host-less launch requires a grid")
     if params is not None and blobs:
@@ -197,3 +200,53 @@ def launch(link_json: str | Path, *, grid: tuple[int, ...] | None, buffers: dict
     g = tuple(grid) + (1,) * (3 - len(grid))
     return {"geometry": {"grid": list(g), "block": [link["threads"], 1, 1], "dynamic_smem_bytes": link["dyn_smem_bytes"]},
             "outputs": {name: str(path) for name, path in (outputs or {}).items()}}
+
+
+def _launch_host(link_path: Path, link: dict[str, Any], providers: dict[str, str], host_inputs, device: int, backend, grid,
+                 buffers, params, blobs) -> dict[str, Any]:
+    """The provider route of ``pipec launch``: report / query / build through the named libraries, one launch, outputs
+    written as raw bytes to the files the inputs name."""
+    import ctypes
+
+    from ..host import broker
+    from ..host.backend import HipBackend, PlkError
+    from ..host.fixture import Fixture, load_inputs
+
+    if not link.get("host"):
+        _fail("L-LAUNCH", "launch.providers", "this link has no host section: it takes --grid / --buffer / --params")
+    if grid is not None or buffers or params is not None or blobs:
+        _fail("L-LAUNCH", "launch.host", "a link with a host section takes --provider and --host-inputs only")
+    if host_inputs is None:
+        _fail("L-LAUNCH", "launch.host_inputs", "a link with a host section needs --host-inputs")
+    groups = link["host"]["groups"]
+    expected = sorted(g["params_group"] for g in groups)
+    if sorted(providers) != expected:
+        _fail("L-HOSTABI", "launch.providers", "provider maps must exactly resolve params groups", expected=expected,
+              actual=sorted(providers))
+    image = (link_path.parent / link["target"]["image"]).read_bytes()
+    libs = {}
+    for group, so in providers.items():
+        try:
+            libs[group] = ctypes.CDLL(str(so))
+        except OSError as err:
+            _fail("L-HOSTABI", f"launch.providers.{group}", f"cannot load provider: {err}")
+    be = backend or HipBackend(device)
+    try:
+        with Fixture(be) as fixture:
+            scalars, output_paths = load_inputs(host_inputs, fixture)
+            resources = {g["owner"]: {c["name"]: fixture.resources[c["name"]] for c in g["channels"] if c["name"] in fixture.resources}
+                         for g in groups}
+            try:
+                with broker.open_host(link, image, resources, scalars, be, providers=libs) as session:
+                    session.launch()
+                    be.synchronize()
+                    geometry = session.geometry
+            except PlkError as err:
+                _fail("L-HOSTABI", "launch.host", str(err))
+            for name, data in fixture.readback().items():
+                output_paths[name].write_bytes(data)
+    finally:
+        if backend is None:
+            be.close()
+    return {"geometry": {"grid": list(geometry["grid"]), "block": list(geometry["block"]), "dynamic_smem_bytes": geometry["dyn_lds"]},
+            "outputs": {name: str(path) for name, path in output_paths.items()}}

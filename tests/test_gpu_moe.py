@@ -242,6 +242,54 @@ def test_broker_route_gives_the_same_bytes_as_the_forward_entry(cell):
     assert torch.equal(t["y"].cpu().view(torch.int16), want[2].view(torch.int16))
 
 
+def test_launch_verb_runs_both_passes_through_the_providers(cell, tmp_path):
+    """`pipec launch LINK --provider GROUP=SO ... --host-inputs JSON` (cli.py:226-258 in the reference): buffers from
+    files, one launch per invocation, outputs written back to files -- against the forward entry's bytes."""
+    import json
+    from pipelink_amd.host import mok_inputs
+    from pipelink_amd.host.backend import LIB_PATH
+    from pipelink_amd.host.mok import scale_pitch, weight_codes_to_k64_tiled, weight_scales_to_slot_major
+    from pipelink_amd.pipec import cli
+    from pipelink_amd.stages.mok import build as mok_build
+
+    T, H, I, E, k = 300, 320, 192, 4, 2
+    inp = mok_inputs.generate(T, H, I, E, k, seed=1)
+    want = _run(cell[0], inp, H, I)
+    dev = torch.device("cuda:0")
+    d = {n: v.to(dev) for n, v in inp.__dict__.items()}
+    t = dict(x_q=d["x_q"], x_sc=d["x_sc"], row_token=d["row_token"], tokens_per_expert=d["tokens_per_expert"],
+             w_gate_q=weight_codes_to_k64_tiled(d["w_gate_q"], H), w_gate_sc=weight_scales_to_slot_major(d["w_gate_sc"], H),
+             w_up_q=weight_codes_to_k64_tiled(d["w_up_q"], H), w_up_sc=weight_scales_to_slot_major(d["w_up_sc"], H),
+             w_down_q=weight_codes_to_k64_tiled(d["w_down_q"], I), w_down_sc=weight_scales_to_slot_major(d["w_down_sc"], I))
+    rows = int(inp.tokens_per_expert.sum())
+    resources = {}
+    for name, tensor in t.items():
+        data = tensor.cpu().contiguous().numpy().tobytes()
+        (tmp_path / f"{name}.bin").write_bytes(data)
+        resources[name] = {"data": f"{name}.bin", "allocation_bytes": len(data)}
+    sizes = {"hidden_q": rows * I, "hidden_sc": rows * scale_pitch(I), "y": rows * H * 2}
+    scalars = {"mok.num_local_tokens": T, "mok.hidden": H, "mok.intermediate": I, "mok.num_local_experts": E,
+               "mok.swiglu_limit": 7.0, "mok.pass": 1, "mok.precision": 1, "mok.routed_rows": rows, "mok.ld_q_h": H,
+               "mok.ld_q_i": I, "mok.ld_sc_h": scale_pitch(H), "mok.ld_sc_i": scale_pitch(I)}
+    link = str(mok_build.images()["link_json"])
+    providers = [arg for g in ("mok.framework.params", "mok.gemm.params", "mok.act.params") for arg in ("--provider", f"{g}={LIB_PATH}")]
+    first = dict(resources, hidden_q={"data": None, "allocation_bytes": sizes["hidden_q"], "output": "hidden_q.bin"},
+                 hidden_sc={"data": None, "allocation_bytes": sizes["hidden_sc"], "output": "hidden_sc.bin"},
+                 y={"data": None, "allocation_bytes": sizes["y"]})
+    (tmp_path / "pass1.json").write_text(json.dumps({"scalars": scalars, "resources": first}))
+    assert cli.main(["launch", link, *providers, "--host-inputs", str(tmp_path / "pass1.json")]) == 0
+    hq = np.frombuffer((tmp_path / "hidden_q.bin").read_bytes(), np.uint8).reshape(rows, I)
+    hsc = np.frombuffer((tmp_path / "hidden_sc.bin").read_bytes(), np.uint8).reshape(rows, scale_pitch(I))
+    assert np.array_equal(hq, want[0]) and np.array_equal(hsc[:, :I // 32], want[1][:, :I // 32])   # the pitch's padding is not written
+    second = dict(resources, hidden_q={"data": "hidden_q.bin", "allocation_bytes": sizes["hidden_q"]},
+                  hidden_sc={"data": "hidden_sc.bin", "allocation_bytes": sizes["hidden_sc"]},
+                  y={"data": None, "allocation_bytes": sizes["y"], "output": "y.bin"})
+    (tmp_path / "pass2.json").write_text(json.dumps({"scalars": dict(scalars, **{"mok.pass": 2}), "resources": second}))
+    assert cli.main(["launch", link, *providers, "--host-inputs", str(tmp_path / "pass2.json")]) == 0
+    y = np.frombuffer((tmp_path / "y.bin").read_bytes(), np.int16).reshape(rows, H)
+    assert np.array_equal(y, want[2].view(torch.int16).numpy())
+
+
 def test_forward_captured_in_a_graph_replays_to_the_same_bytes(cell):
     """HipBackend.capture / Graph.launch (the reference's CudaBackend.capture, host/cuda.py:267-286): the forward's
     two launches and a fill recorded on a created stream, replayed three times with eager work and

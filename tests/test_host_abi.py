@@ -213,3 +213,53 @@ def test_fixture_owns_buffers_until_it_closes():
         fx.tensor("a", data=None, allocation_bytes=4)
     assert lost.freed == []                                           # an abandoned backend's memory is not reused
     assert Domain(0, 1).world == 1
+
+
+def test_launch_verb_takes_a_host_link_through_its_providers(tmp_path):
+    """`pipec launch` on a link with a host section (cli.py:226-258, launcher.py:284-333 in the reference): the
+    argument checks that need no GPU."""
+    from pipelink_amd.pipec import cli, launcher
+    from pipelink_amd.pipec.clauses import LaunchError
+    from pipelink_amd.host.fixture import Fixture, load_inputs
+
+    link_path = os.path.join(ROOT, "pipelink_amd", "stages", "mok", "build", "link", "link.json")
+    with pytest.raises(LaunchError) as err:
+        launcher.launch(link_path, grid=(8,))
+    assert err.value.failures[0].path == "launch.host"                        # host-less arguments on a host link
+    with pytest.raises(LaunchError) as err:
+        launcher.launch(link_path, grid=None, providers={"mok.gemm.params": "x.so"})
+    assert err.value.failures[0].path == "launch.host_inputs"
+    inputs = tmp_path / "inputs.json"
+    inputs.write_text(json.dumps({"scalars": {}, "resources": {}}))
+    with pytest.raises(LaunchError) as err:
+        launcher.launch(link_path, grid=None, providers={"mok.gemm.params": "x.so"}, host_inputs=inputs)
+    assert err.value.clause_ids == {"L-HOSTABI"} and err.value.failures[0].detail["expected"] == [
+        "mok.act.params", "mok.framework.params", "mok.gemm.params"]
+    assert cli.main(["launch", link_path, "--provider", "mok.gemm.params=x.so", "--host-inputs", str(inputs)]) == 1
+
+    class Memory:
+        lost = False
+        def __init__(self): self.mem, self.next = {}, 0x1000
+        def allocate(self, size, align=256):
+            addr, self.next = self.next, self.next + (size + 255) // 256 * 256
+            self.mem[addr] = bytearray(size)
+            return addr
+        def free(self, addr): pass
+        def upload(self, addr, data, stream=None): self.mem[addr][:len(data)] = data
+        def zero(self, addr, size, stream=None): pass
+        def readback(self, addr, size, stream=None): return bytes(self.mem[addr][:size])
+        def synchronize(self, stream=None): pass
+
+    (tmp_path / "x.bin").write_bytes(b"\x05" * 16)
+    inputs.write_text(json.dumps({"scalars": {"mok.hidden": 64}, "resources": {
+        "x_q": {"data": "x.bin", "allocation_bytes": 16, "extents": [1, 16], "bit_strides": [128, 8], "dtype_id": 1, "alignment": 16,
+                "origin_byte_offset": 0, "origin_bit_offset": 0},
+        "y": {"data": None, "allocation_bytes": 32, "output": "y.bin"}}}))
+    with Fixture(Memory()) as fx:
+        scalars, outputs = load_inputs(inputs, fx)
+        assert scalars == {"mok.hidden": 64} and outputs == {"y": tmp_path / "y.bin"}
+        assert fx.resources["x_q"].allocation_bytes == 16 and fx.backend.mem[fx.resources["x_q"].address] == b"\x05" * 16
+        assert set(fx.readback()) == {"y"}
+    inputs.write_text(json.dumps({"scalars": {}, "resources": {"x_q": {"data": None}}}))
+    with pytest.raises(ValueError), Fixture(Memory()) as fx:
+        load_inputs(inputs, fx)
