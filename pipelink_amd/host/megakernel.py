@@ -1,6 +1,7 @@
 """Host side of the decode megakernel example on the host-less route: one launch = one decoded token."""
 from __future__ import annotations
 
+import json
 from pathlib import Path
 
 import numpy as np
@@ -28,7 +29,8 @@ def open_session(link_json: str | Path, weights: np.ndarray, kv_cache: np.ndarra
         raise ValueError("the attention output and the chunk weights do not fit the workgroup's LDS vector")
     if (pos + chunks - 1) // chunks + 1 > 8192 + 256 - 1280:  # the scores sit 1280 floats into the vector
         raise ValueError("a context chunk does not fit the workgroup's LDS vector: use more workgroups")
-    prog = mk.program(layers)
+    link = json.loads(Path(link_json).read_text()) if not isinstance(link_json, dict) else link_json
+    prog = mk.program(layers, mk.opcodes_of(link))   # the instruction stream speaks the numbers this link bound
     buffers = {"weights": weights, "kv_cache": kv_cache, "x": x.astype(np.float32), "rope": mk.rope_table(pos), "program": prog,
                "qkv": (((hq + 2 * hkv) * mk.HEAD_DIM,), np.float32), "attn_partial": ((hq * chunks * mk.PARTIAL_STRIDE,), np.float32),
                "h": ((dff,), np.float32), "logits": ((vocab,), np.float32), "sync": ((512,), np.uint32)}

@@ -47,7 +47,9 @@ GFX950 = Profile(
     max_waves_per_workgroup=16, simds_per_cu=4, regs_per_lane=512, reg_granule=8,
     param_limit_bytes=4096, named_barriers=1,
     domains={"smem": ("smem", 1), "mbarrier": ("smem", 16), "warp": ("warp", 1),
-             "named_barrier": ("named_barrier", 1), "gmem_counter": ("gmem_counter", 1)},
+             "named_barrier": ("named_barrier", 1), "gmem_counter": ("gmem_counter", 1),
+             # numbers an interpreter dispatches on; capacity comes from the pipeline (profile.py:119-126 in the reference)
+             "opcode": ("opcode", 1)},
 )
 
 # The reference's own profile names are accepted when its fixtures are loaded: the checks that

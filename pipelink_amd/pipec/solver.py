@@ -82,6 +82,9 @@ def _align_up(x: int, a: int) -> int:
     return (x + a - 1) // a * a
 
 
+PIPELINE_SIZED = ("gmem_counter", "opcode")
+
+
 def _first_fit(order, placed: list[Interval], pairs, capacity):
     """Place claims in the given order; returns (high water, intervals) or None."""
     out = list(placed)
@@ -238,7 +241,7 @@ def solve(pipeline: Pipeline, stages: list[Stage], expansions: list[Expansion] |
                 life = c.get("lifetime", "kernel")
                 per_phys.setdefault(phys[0], []).append({
                     "handle": c["handle"], "domain": c["domain"], "physical": phys[0], "unit": phys[1],
-                    "size": extent * phys[1], "align": c.get("align", 1), "fixed": c.get("at"),
+                    "size": extent * phys[1], "align": c.get("align", 1), "fixed": forced.get(c["handle"], c.get("at")),
                     "phase": "kernel" if life == "kernel" else life[6:], "stage": s.id})
         if bad:
             blocked.add(bad)
@@ -247,8 +250,8 @@ def solve(pipeline: Pipeline, stages: list[Stage], expansions: list[Expansion] |
         feasible = True
         for phys, claims in sorted(per_phys.items()):
             cap = prof.capacity(phys)
-            if phys == "gmem_counter":
-                cap = (body.get("domains", {}).get("gmem_counter") or {}).get("capacity")
+            if phys in PIPELINE_SIZED:  # storage the pipeline sizes, not the chip
+                cap = (body.get("domains", {}).get(phys) or {}).get("capacity")
             res = _pack(claims, pairs, cap)
             if res is None:
                 feasible = False
@@ -261,7 +264,7 @@ def solve(pipeline: Pipeline, stages: list[Stage], expansions: list[Expansion] |
         for phys, ivs in intervals.items():
             for iv in ivs:
                 unit = prof.physical(iv.domain)[1]
-                bindings[iv.handle] = (iv.lo // unit, "solved")
+                bindings[iv.handle] = (iv.lo // unit, "forced" if iv.handle in forced else "solved")
         for s, c in warp_claims:
             first = min(role_warps[r][1] for r in c.get("roles", [])) if c.get("roles") else 0
             bindings[c["handle"]] = (first, "solved")

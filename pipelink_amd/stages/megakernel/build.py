@@ -4,7 +4,8 @@ persistent gfx950 kernel, builds the one-unit control, then swaps ONLY the atten
 
 Counterpart of campaigns/megakernel/port/build.sh in the reference (interpreter + op packages, relink
 with another attention).  Output under ``build/``: the ``.plink`` packages, ``pipeline.json``,
-``link/...``, ``one_unit.hsaco``, and ``swap/{pipeline.json, link/...}``."""
+``link/...``, ``one_unit.hsaco``, ``swap/{pipeline.json, link/...}`` and ``rebind/{pipeline.json, link/...}`` (the
+same packages linked with other opcode numbers, campaigns/megakernel/port/pipelines/rebind-opcode.json)."""
 from __future__ import annotations
 
 import json
@@ -37,15 +38,22 @@ def build(out: Path = BUILD, one_unit: bool = True) -> dict:
         shutil.copy(f, swap / f.name)
     (swap / "pipeline.json").write_text((HERE / "pipeline_attn_wide.json").read_text())
     swapped = linker.link(swap / "pipeline.json", swap / "link")
-    for d in (out, out / "link", swap, swap / "link"):
+    rebind = out / "rebind"   # the same packages, other opcode numbers: only the pipeline's forced bindings differ
+    rebind.mkdir(exist_ok=True)
+    for f in out.glob("*.plink"):
+        shutil.copy(f, rebind / f.name)
+    (rebind / "pipeline.json").write_text((HERE / "pipeline_rebind_opcodes.json").read_text())
+    rebound = linker.link(rebind / "pipeline.json", rebind / "link")
+    for d in (out, out / "link", swap, swap / "link", rebind, rebind / "link"):
         for junk in d.glob("*.bc"):
             junk.unlink()
-    return {"packages": reports, "link": link, "one_unit": control, "swap": swapped}
+    return {"packages": reports, "link": link, "one_unit": control, "swap": swapped, "rebind": rebound}
 
 
 def images(out: Path = BUILD) -> dict:
     paths = {"link_json": out / "link" / "link.json", "linked": out / "link" / "pipeline.hsaco", "one_unit": out / "one_unit.hsaco",
-             "swap_link_json": out / "swap" / "link" / "link.json", "swap_linked": out / "swap" / "link" / "pipeline.hsaco"}
+             "swap_link_json": out / "swap" / "link" / "link.json", "swap_linked": out / "swap" / "link" / "pipeline.hsaco",
+             "rebind_link_json": out / "rebind" / "link" / "link.json", "rebind_linked": out / "rebind" / "link" / "pipeline.hsaco"}
     missing = [str(p) for p in paths.values() if not p.exists()]
     if missing:
         raise FileNotFoundError("megakernel example is not built (run __graft_entry__.build()): " + ", ".join(missing))

@@ -23,17 +23,17 @@
 // units), its sum of exponentials, two floats of padding (rows stay 16-byte aligned)
 #define MK_PARTIAL_STRIDE (MK_HEAD_DIM + 4)
 
-enum {
-  MK_OP_RMSNORM_ATTN = 1, /* x * rsqrt(mean x^2 + eps) * attn_norm[layer]  -> LDS vector */
-  MK_OP_QKV = 2,          /* qkv = Wqkv[layer] . vector */
-  MK_OP_ATTN = 3,         /* RoPE, append to the cache, partial attention of (head, chunk) */
-  MK_OP_OPROJ = 4,        /* combine the partials; x += Wo[layer] . attention */
-  MK_OP_RMSNORM_FFN = 5,
-  MK_OP_UPGATE = 6,       /* h = silu(Wgate . vector) * (Wup . vector) */
-  MK_OP_DOWN = 7,         /* x += Wdown . h */
-  MK_OP_RMSNORM_FINAL = 8,
-  MK_OP_LMHEAD = 9        /* logits = Wlm . vector */
-};
+/* Opcodes are not constants of this header: each op package claims one number in the link's "opcode" domain
+ * (pipelink_mk_opcode_<op>), the pipeline binds the numbers, the interpreter and the ops read them through the
+ * handle functions, and the host takes them from link.json ("bindings") when it writes the instruction stream.
+ * An opcode nobody claimed is a no-op.  The ops:
+ *   rmsnorm_attn   x * rsqrt(mean x^2 + eps) * attn_norm[layer]  -> LDS vector      (rmsnorm_ffn, rmsnorm_final alike)
+ *   qkv            qkv = Wqkv[layer] . vector
+ *   attn           RoPE, append to the cache, partial attention of (head, chunk)
+ *   oproj          combine the partials; x += Wo[layer] . attention
+ *   upgate         h = silu(Wgate . vector) * (Wup . vector)
+ *   down           x += Wdown . h
+ *   lmhead         logits = Wlm . vector */
 
 /* one instruction: 4 x int32 */
 typedef struct MkInstr {

@@ -18,6 +18,17 @@ extern "C" __device__ void pipelink_call_op_upgate(const void* view, const MkIns
 extern "C" __device__ void pipelink_call_op_down(const void* view, const MkInstr* instr);
 extern "C" __device__ void pipelink_call_op_lmhead(const void* view, const MkInstr* instr);
 
+// the opcode numbers the link bound to the op packages' claims
+extern "C" __device__ int pipelink_mk_opcode_rmsnorm_attn();
+extern "C" __device__ int pipelink_mk_opcode_qkv();
+extern "C" __device__ int pipelink_mk_opcode_attn();
+extern "C" __device__ int pipelink_mk_opcode_oproj();
+extern "C" __device__ int pipelink_mk_opcode_rmsnorm_ffn();
+extern "C" __device__ int pipelink_mk_opcode_upgate();
+extern "C" __device__ int pipelink_mk_opcode_down();
+extern "C" __device__ int pipelink_mk_opcode_rmsnorm_final();
+extern "C" __device__ int pipelink_mk_opcode_lmhead();
+
 namespace mk_interp {
 constexpr uint32_t SPIN_LIMIT = 1u << 22;
 
@@ -77,18 +88,15 @@ extern "C" __device__ void mk_interp_role_worker(const void* params, unsigned va
   uint32_t passed = 0;
   for (int i = 0; i < m.num_instr; ++i) {
     const MkInstr* instr = m.program + i;
-    switch (instr->opcode) {  // uniform over the grid
-      case MK_OP_RMSNORM_ATTN:
-      case MK_OP_RMSNORM_FFN:
-      case MK_OP_RMSNORM_FINAL: pipelink_call_op_rmsnorm(&view, instr); break;
-      case MK_OP_QKV: pipelink_call_op_qkv(&view, instr); break;
-      case MK_OP_ATTN: pipelink_call_op_attn(&view, instr); break;
-      case MK_OP_OPROJ: pipelink_call_op_oproj(&view, instr); break;
-      case MK_OP_UPGATE: pipelink_call_op_upgate(&view, instr); break;
-      case MK_OP_DOWN: pipelink_call_op_down(&view, instr); break;
-      case MK_OP_LMHEAD: pipelink_call_op_lmhead(&view, instr); break;
-      default: break;
-    }
+    const int op = instr->opcode;  // uniform over the grid; the numbers are bound at link time
+    if (op == pipelink_mk_opcode_rmsnorm_attn() || op == pipelink_mk_opcode_rmsnorm_ffn() || op == pipelink_mk_opcode_rmsnorm_final())
+      pipelink_call_op_rmsnorm(&view, instr);
+    else if (op == pipelink_mk_opcode_qkv()) pipelink_call_op_qkv(&view, instr);
+    else if (op == pipelink_mk_opcode_attn()) pipelink_call_op_attn(&view, instr);
+    else if (op == pipelink_mk_opcode_oproj()) pipelink_call_op_oproj(&view, instr);
+    else if (op == pipelink_mk_opcode_upgate()) pipelink_call_op_upgate(&view, instr);
+    else if (op == pipelink_mk_opcode_down()) pipelink_call_op_down(&view, instr);
+    else if (op == pipelink_mk_opcode_lmhead()) pipelink_call_op_lmhead(&view, instr);
     if (instr->barrier_after) mk_interp::grid_barrier(m, passed);
     else __syncthreads();  // the next op of this workgroup reads what this one left in LDS
   }
@@ -128,5 +136,14 @@ MK_CALL(lmhead);
 // the ops' reduction scratch
 PL_CLAIM("pipelink_mk_vec", "smem", 33792, 1024, "kernel");
 PL_USES("pipelink_mk_vec");
+PL_USES("pipelink_mk_opcode_rmsnorm_attn");
+PL_USES("pipelink_mk_opcode_qkv");
+PL_USES("pipelink_mk_opcode_attn");
+PL_USES("pipelink_mk_opcode_oproj");
+PL_USES("pipelink_mk_opcode_rmsnorm_ffn");
+PL_USES("pipelink_mk_opcode_upgate");
+PL_USES("pipelink_mk_opcode_down");
+PL_USES("pipelink_mk_opcode_rmsnorm_final");
+PL_USES("pipelink_mk_opcode_lmhead");
 PL_PRELUDE("include/mk_abi.h");
 PL_EMIT_MAIN()

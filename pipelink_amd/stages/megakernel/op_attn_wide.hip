@@ -125,5 +125,7 @@ PL_EXPORT(op_attn, mk_attn_wide_op, "extern \"C\" __device__ void mk_attn_wide_o
 PL_SERVE(op_attn, "op_attn");
 PL_CALL(rope_apply, "rope_apply", "extern \"C\" __device__ float pipelink_call_rope_apply(const void* view, const float* v, int i);");
 PL_USES("pipelink_mk_vec");
+// the number(s) the instruction stream calls this op by: one slot each in the link's opcode domain
+PL_CLAIM("pipelink_mk_opcode_attn", "opcode", 1, 1, "kernel");
 PL_PRELUDE("include/mk_abi.h");
 PL_EMIT_MAIN()

@@ -4,11 +4,14 @@
 #ifndef PIPELINK_EMIT
 #include "mk_device.hpp"
 
+extern "C" __device__ int pipelink_mk_opcode_rmsnorm_ffn();
+extern "C" __device__ int pipelink_mk_opcode_rmsnorm_final();
+
 extern "C" __device__ void mk_rmsnorm_op(const void* view, const MkInstr* instr) {
   const MkModel& m = mk::model(view);
-  const uint16_t* weight = instr->opcode == MK_OP_RMSNORM_FINAL ? mk::final_norm(m)
-                           : instr->opcode == MK_OP_RMSNORM_FFN ? mk::layer_of(m, instr->layer).ffn_norm
-                                                                : mk::layer_of(m, instr->layer).attn_norm;
+  const uint16_t* weight = instr->opcode == pipelink_mk_opcode_rmsnorm_final() ? mk::final_norm(m)
+                           : instr->opcode == pipelink_mk_opcode_rmsnorm_ffn() ? mk::layer_of(m, instr->layer).ffn_norm
+                                                                               : mk::layer_of(m, instr->layer).attn_norm;
   float* out = mk::vec();
   float* scratch = out + m.d;  // 4 floats behind the vector (the vector region holds at least D + 64 floats)
   const int tid = threadIdx.x;
@@ -35,5 +38,11 @@ PL_VARIANT(0, {});
 PL_EXPORT(op_rmsnorm, mk_rmsnorm_op, "extern \"C\" __device__ void mk_rmsnorm_op(const void* view, const MkInstr* instr);");
 PL_SERVE(op_rmsnorm, "op_rmsnorm");
 PL_USES("pipelink_mk_vec");
+PL_USES("pipelink_mk_opcode_rmsnorm_ffn");
+PL_USES("pipelink_mk_opcode_rmsnorm_final");
+// the number(s) the instruction stream calls this op by: one slot each in the link's opcode domain
+PL_CLAIM("pipelink_mk_opcode_rmsnorm_attn", "opcode", 1, 1, "kernel");
+PL_CLAIM("pipelink_mk_opcode_rmsnorm_ffn", "opcode", 1, 1, "kernel");
+PL_CLAIM("pipelink_mk_opcode_rmsnorm_final", "opcode", 1, 1, "kernel");
 PL_PRELUDE("include/mk_abi.h");
 PL_EMIT_MAIN()

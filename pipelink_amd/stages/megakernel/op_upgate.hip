@@ -33,5 +33,7 @@ PL_VARIANT(0, {});
 PL_EXPORT(op_upgate, mk_upgate_op, "extern \"C\" __device__ void mk_upgate_op(const void* view, const MkInstr* instr);");
 PL_SERVE(op_upgate, "op_upgate");
 PL_USES("pipelink_mk_vec");
+// the number(s) the instruction stream calls this op by: one slot each in the link's opcode domain
+PL_CLAIM("pipelink_mk_opcode_upgate", "opcode", 1, 1, "kernel");
 PL_PRELUDE("include/mk_abi.h");
 PL_EMIT_MAIN()

@@ -9,13 +9,23 @@ HEAD_DIM = 64
 PARTIAL_STRIDE = HEAD_DIM + 4  # MK_PARTIAL_STRIDE
 
 
-def program(layers: int) -> np.ndarray:
-    """[n, 4] int32 (opcode, layer, barrier_after, 0): the whole decoding step."""
+OPS = ("rmsnorm_attn", "qkv", "attn", "oproj", "rmsnorm_ffn", "upgate", "down", "rmsnorm_final", "lmhead")
+DEFAULT_OPCODES = dict(zip(OPS, range(1, 10)))
+
+
+def opcodes_of(link: dict) -> dict[str, int]:
+    """op name -> the number the link bound to its claim (link.json "bindings": pipelink_mk_opcode_<op>)."""
+    return {op: link["bindings"][f"pipelink_mk_opcode_{op}"][0] for op in OPS}
+
+
+def program(layers: int, opcodes: dict[str, int] | None = None) -> np.ndarray:
+    """[n, 4] int32 (opcode, layer, barrier_after, 0): the whole decoding step, in the opcode numbers of one link."""
+    n = opcodes or DEFAULT_OPCODES
     rows = []
     for l in range(layers):
-        rows += [(OP_RMSNORM_ATTN, l, 0), (OP_QKV, l, 1), (OP_ATTN, l, 1), (OP_OPROJ, l, 1),
-                 (OP_RMSNORM_FFN, l, 0), (OP_UPGATE, l, 1), (OP_DOWN, l, 1)]
-    rows += [(OP_RMSNORM_FINAL, 0, 0), (OP_LMHEAD, 0, 0)]
+        rows += [(n["rmsnorm_attn"], l, 0), (n["qkv"], l, 1), (n["attn"], l, 1), (n["oproj"], l, 1),
+                 (n["rmsnorm_ffn"], l, 0), (n["upgate"], l, 1), (n["down"], l, 1)]
+    rows += [(n["rmsnorm_final"], 0, 0), (n["lmhead"], 0, 0)]
     return np.array([(o, l, b, 0) for o, l, b in rows], dtype=np.int32)
 
 

@@ -85,6 +85,36 @@ def test_links_nine_packages_and_swaps_only_the_attention(example):
     assert "mk.attn" in link["input_hashes"] and "mk.attn.wide" in swap["input_hashes"]
 
 
+@needs_rocm
+def test_opcodes_are_bound_at_link_time(example):
+    """The op packages claim slots of the link's opcode domain; the pipeline binds the numbers; a relink with other
+    numbers reuses every package (campaigns/megakernel/port/pipelines/{a,rebind-opcode}.json in the reference)."""
+    out, res = example
+    link, rebind = res["link"], res["rebind"]
+    assert mkp.opcodes_of(link) == mkp.DEFAULT_OPCODES
+    assert all(link["bindings"][f"pipelink_mk_opcode_{op}"][1] == "forced" for op in mkp.OPS)
+    other = mkp.opcodes_of(rebind)
+    assert sorted(other.values()) != sorted(mkp.DEFAULT_OPCODES.values()) and len(set(other.values())) == 9
+    assert rebind["input_hashes"] == link["input_hashes"]                       # not one package was repacked
+    assert [iv["handle"] for iv in link["intervals"]["opcode"]] == [f"pipelink_mk_opcode_{op}" for op in mkp.OPS]
+    assert list(mkp.program(1, other)[:3, 0]) == [other["rmsnorm_attn"], other["qkv"], other["attn"]]
+    # two ops bound to one number: the claims overlap
+    from pipelink_amd.pipec import linker
+    from pipelink_amd.pipec.clauses import PipeLinkError
+    clash = json.loads((out / "pipeline.json").read_text())
+    clash["pipeline"]["forced_bindings"]["pipelink_mk_opcode_down"] = clash["pipeline"]["forced_bindings"]["pipelink_mk_opcode_qkv"]
+    (out / "clash.json").write_text(json.dumps(clash))
+    with pytest.raises(PipeLinkError) as err:
+        linker.link(out / "clash.json", out / "clash", codegen=False)
+    assert "L-OVERLAP" in err.value.clause_ids
+    # a number past the domain's capacity
+    clash["pipeline"]["forced_bindings"]["pipelink_mk_opcode_down"] = 16
+    (out / "clash.json").write_text(json.dumps(clash))
+    with pytest.raises(PipeLinkError) as err:
+        linker.link(out / "clash.json", out / "clash", codegen=False)
+    assert "L-OVERLAP" in err.value.clause_ids
+
+
 # ---- GPU ---------------------------------------------------------------------------------------------------
 
 def _bits(t: torch.Tensor) -> np.ndarray:
@@ -131,6 +161,8 @@ def test_small_model_matches_the_oracle_linked_one_unit_and_swapped():
     assert np.array_equal(got["kv_cache"][:, :, :37], _bits(cache)[:, :, :37])  # the rest of the cache untouched
     control = _run("link_json", cfg, weights, cache, x, workgroups=32, image_key="one_unit")
     assert all(np.array_equal(control[n], got[n]) for n in ("logits", "x", "kv_cache")), "linked and one-unit images differ"
+    rebound = _run("rebind_link_json", cfg, weights, cache, x, workgroups=32)   # other opcode numbers, same packages
+    assert all(np.array_equal(rebound[n], got[n]) for n in ("logits", "x", "kv_cache")), "rebound opcodes changed the result"
     swapped = _run("swap_link_json", cfg, weights, cache, x, workgroups=32)
     assert list(swapped["sync"][:3]) == [0, 0, 0]
     assert _rel(swapped["logits"], got["logits"]) <= 1e-4 and _rel(swapped["logits"], want_logits.numpy()) <= 2e-3
