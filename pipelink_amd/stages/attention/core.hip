@@ -7,8 +7,8 @@
 // is only a summation order, and V^T is read from LDS in the order the registers hold the keys:
 //   group g of 16 keys (registers 8g .. 8g+7 of a 32-key score tile), lane half h = lane / 32:
 //   elements 0-3 = keys 16g + 4h + 0..3, elements 4-7 = keys 16g + 8 + 4h + 0..3.
-// K and V both go global -> LDS as stored (row-major [key][d], 16-byte chunks swizzled by position =
-// chunk ^ (key % 16)).  K rows are the A operand of the first product as they are.  The A operand of the
+// K and V both go global -> LDS as stored (row-major [key][d], the 16-byte chunks of a row permuted so that the
+// reads below meet no bank conflict: k_place / v_place).  K rows are the A operand of the first product as they are.  The A operand of the
 // second product wants, per lane, four consecutive KEYS at one d -- a column of the V tile: that is what
 // ds_read_b64_tr_b16 delivers.  In a group of 16 lanes, lane i hands in the address of 4 consecutive d
 // (8 bytes) and lane j receives element j % 4 of the data of lanes j / 4, j / 4 + 4, j / 4 + 8, j / 4 + 12
@@ -44,20 +44,37 @@ typedef short v4s __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4s* lds_v4s;
 constexpr float MASKED = -1.0e30f;
 
+// Where the 16-byte chunk `chunk` of a key's row stands in its 256-byte LDS row.  K is read one key per lane, 16 lanes
+// = 16 consecutive keys at one chunk: the 16 rows must put that chunk in 16 different places.  V is read in columns,
+// 32 lanes = 4 consecutive keys x 4 consecutive chunks: the 4 rows must put each group of 4 chunks in a different place.
+__device__ __forceinline__ int k_place(int key, int chunk) { return chunk ^ (key & 15); }
+__device__ __forceinline__ int v_place(int key, int chunk) { return chunk ^ (4 * (key & 3)); }
+
 // one 64-key block of K or V -> LDS: 64 keys x 256 B; one load instruction of a wave moves 4 keys (1 KB)
+template <bool IS_V>
 __device__ __forceinline__ void issue_block(__amdgpu_buffer_rsrc_t src, uint32_t first_key_byte, unsigned char* dst, int wave, int lane) {
   const int kr = lane >> 4, pos = lane & 15;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int key = (wave * 4 + j) * 4 + kr;  // 0..63
-    const uint32_t off = first_key_byte + (uint32_t)key * (FA_D * 2) + 16u * (uint32_t)(pos ^ (key & 15));
+    const uint32_t off = first_key_byte + (uint32_t)key * (FA_D * 2) + 16u * (uint32_t)(IS_V ? v_place(key, pos) : k_place(key, pos));
     __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (lds_ptr)(dst + (wave * 4 + j) * 1024), 16, (int)off, 0, 0, 0);
   }
 }
-// 4 consecutive keys from `key` on, at the d this lane's group position stands for (see the head of the file)
-__device__ __forceinline__ v4s read_v_column(const unsigned char* vbuf, int key, int d) {
-  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-      (lds_v4s)(const_cast<unsigned char*>(vbuf) + key * (FA_D * 2) + 16 * ((d >> 3) ^ (key & 15)) + 2 * (d & 4)));
+// The transposing read: in a group of 16 lanes, lane i hands in the address of 4 consecutive d of key kbase + i / 4
+// and lane j receives keys kbase .. kbase + 3 at d = dbase + j.
+__device__ __forceinline__ v4s read_v_piece(const unsigned char* at) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(const_cast<unsigned char*>(at)));
+}
+// A value of this lane and the one of lane ^ 32, without a trip through the LDS: after the swap the first result
+// holds the lower half-wave's values in both halves, the second the upper half-wave's.
+__device__ __forceinline__ float max_with_other_half(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_with_other_half(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 }  // namespace fa_core
 
@@ -99,31 +116,65 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
   const int keys = pipelink_call_mask_key_count(&view, q0, q0 + FA_Q_TILE - 1);
   const int blocks = (keys + FA_K_BLOCK - 1) / FA_K_BLOCK;
   const int wave_keys = pipelink_call_mask_key_count(&view, qw, qw + 31);
-  issue_block(kres, 0u, buf, wave, lane);
-  issue_block(vres, 0u, buf + K_BYTES, wave, lane);
+  // Schedule.  Two LDS buffers per operand: block i + 1 is in flight while block i is multiplied; one barrier per
+  // block.  LDS reads are issued in batches ahead of the MFMAs that use them (a read costs a few hundred clocks of
+  // latency, an MFMA 32): all 16 K fragments of a block before its first score MFMA, the V pieces of the next group
+  // of 16 keys before the MFMAs of the present one, those of the first group before the softmax.
   const int li = lane & 15, dgroup = 16 * ((lane >> 4) & 1);  // position in the 16-lane group, the group's first d in a 32-row block
+  // LDS addresses, kept few: a K fragment is at [key = 32 t + l32][chunk 2 kk + half] -> this lane's 8 places in
+  // its row (the tile t is an immediate offset); a V column piece is at [key][chunk 4 db + c] -> 4 places per lane.
+  int k_at[8];
+#pragma unroll
+  for (int kk = 0; kk < 8; ++kk) k_at[kk] = l32 * (FA_D * 2) + 16 * k_place(l32, 2 * kk + half);
+  const int v_key = 4 * half + (li >> 2);  // the key (within a group of 16) this lane points at for the transposing read
+  int v_at[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db) {
+    const int d = 32 * db + dgroup + 4 * (li & 3);
+    v_at[db] = v_key * (FA_D * 2) + 16 * v_place(v_key, d >> 3) + 2 * (d & 4);
+  }
+  // the 8 pieces (4 blocks of d x two halves of 8 keys) of the group of 16 keys that starts at key `first`
+  auto read_v_group = [&](const unsigned char* vbuf, int first, v4s (&piece)[8]) {
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+      // rows first + v_key and 8 further on: (key & 3) is the same, so is the place in the row
+      piece[2 * db] = read_v_piece(vbuf + v_at[db] + first * (FA_D * 2));
+      piece[2 * db + 1] = read_v_piece(vbuf + v_at[db] + (first + 8) * (FA_D * 2));
+    }
+  };
+  issue_block<false>(kres, 0u, buf, wave, lane);
+  issue_block<true>(vres, 0u, buf + K_BYTES, wave, lane);
   for (int i = 0; i < blocks; ++i) {
     unsigned char* kbuf = buf + (i & 1) * BUF_BYTES;
     const unsigned char* vbuf = kbuf + K_BYTES;
     __syncthreads();  // blocks i of K and V have landed (the barrier drains every wave's loads); buffers of block i - 1 are free
     if (i + 1 < blocks) {
-      issue_block(kres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + ((i + 1) & 1) * BUF_BYTES, wave, lane);
-      issue_block(vres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + ((i + 1) & 1) * BUF_BYTES + K_BYTES, wave, lane);
+      issue_block<false>(kres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + ((i + 1) & 1) * BUF_BYTES, wave, lane);
+      issue_block<true>(vres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + ((i + 1) & 1) * BUF_BYTES + K_BYTES, wave, lane);
     }
     const int k0 = i * FA_K_BLOCK;
     if (k0 >= wave_keys) continue;  // no query of this wave sees a key this far on: only the loads and the barrier
     // ---- S^T = K . Q^T : two 32-key tiles -----------------------------------------------------------
     v16f s[2];
+    v4s piece[2][8];
+    {
+      v4i kf[2][8];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[t][r] = 0.0f;
-      const int key = 32 * t + l32;
+        for (int kk = 0; kk < 8; ++kk) kf[t][kk] = *reinterpret_cast<const v4i*>(kbuf + k_at[kk] + t * 32 * (FA_D * 2));
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(2);
 #pragma unroll
-      for (int kk = 0; kk < 8; ++kk) {
-        const v4i raw = *reinterpret_cast<const v4i*>(kbuf + key * (FA_D * 2) + 16 * ((2 * kk + half) ^ (key & 15)));
-        s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, raw), qf[kk], s[t], 0, 0, 0);
+      for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[t][r] = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, kf[t][kk]), qf[kk], s[t], 0, 0, 0);
       }
+      read_v_group(vbuf, 0, piece[0]);  // on their way during the softmax
+      __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     // ---- mask, online softmax (in units of log2: exp2(x * scale_log2e - max)) -------------------------------
     const int query = qw + l32;
@@ -142,7 +193,7 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) block_max = fmaxf(block_max, s[t][r]);
-    block_max = fmaxf(block_max, __shfl_xor(block_max, 32));
+    block_max = max_with_other_half(block_max);
     // every query sees key 0, and block 0 comes first: from then on the maximum is a real score, and a
     // masked entry (-1e30) turns into exp2(-huge) = 0 by itself
     const float new_max = fmaxf(row_max, block_max * p.scale_log2e);
@@ -157,7 +208,7 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
         s[t][r] = e;
         block_sum += e;
       }
-    block_sum += __shfl_xor(block_sum, 32);
+    block_sum = sum_with_other_half(block_sum);
     row_sum = row_sum * alpha + block_sum;
     if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {  // once the maxima have settled nothing needs rescaling
 #pragma unroll
@@ -166,24 +217,25 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
         for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
     }
     // ---- O^T += V^T . P^T : four groups of 16 keys, four 32-row blocks of d ----------------------------
+    __builtin_amdgcn_s_setprio(2);
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int gi = 0; gi < 4; ++gi) {
+      const int t = gi >> 1, g = gi & 1;
+      if (gi + 1 < 4) read_v_group(vbuf, 16 * (gi + 1), piece[(gi + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+      v8f pf;
 #pragma unroll
-      for (int g = 0; g < 2; ++g) {
-        v8f pf;
+      for (int e = 0; e < 8; ++e) pf[e] = s[t][8 * g + e];
+      const v8bf pb = __builtin_convertvector(pf, v8bf);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) pf[e] = s[t][8 * g + e];
-        const v8bf pb = __builtin_convertvector(pf, v8bf);
-        const int key = 32 * t + 16 * g + 4 * half + (li >> 2);  // the row this lane points at: its group's first key + li / 4
-#pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          const int d = 32 * db + dgroup + 4 * (li & 3);
-          const v4s lo = read_v_column(vbuf, key, d), hi = read_v_column(vbuf, key + 8, d);
-          const v2i lo2 = __builtin_bit_cast(v2i, lo), hi2 = __builtin_bit_cast(v2i, hi);
-          const v4i raw = {lo2.x, lo2.y, hi2.x, hi2.y};
-          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, raw), pb, o[db], 0, 0, 0);
-        }
+      for (int db = 0; db < 4; ++db) {
+        const v2i lo2 = __builtin_bit_cast(v2i, piece[gi & 1][2 * db]), hi2 = __builtin_bit_cast(v2i, piece[gi & 1][2 * db + 1]);
+        const v4i raw = {lo2.x, lo2.y, hi2.x, hi2.y};
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, raw), pb, o[db], 0, 0, 0);
       }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_s_setprio(0);
   }
   // ---- O[b][query][h][d] = O^T / row_sum, bf16 ------------------------------------------------------------
   const float inv = row_sum > 0.0f ? __builtin_amdgcn_rcpf(row_sum) : 0.0f;

@@ -122,8 +122,12 @@ def test_stated_case_sampled_heads_one_unit_control_and_output_projection():
         control.launch()
         control.synchronize()
         assert np.array_equal(sess.read("o"), o_bits), "linked and one-unit images differ"
-        ms = sess.time(5)
-        print(f"attention: {ms:.3f} ms, {4 * B * HQ * S * S * 128 / 2 / ms / 1e9:.0f} TFLOP/s on causal flop", flush=True)
+        import time
+        start = time.time()
+        while time.time() - start < 1.0:     # the GPU needs about a second of load to reach its sustained clock state
+            sess.time(50)
+        ms = sorted(sess.time(100) for _ in range(3))[1]
+        print(f"attention: {ms:.3f} ms sustained, {4 * B * HQ * S * S * 128 / 2 / ms / 1e9:.0f} TFLOP/s on causal flop", flush=True)
     finally:
         sess.close()
     o = _from_bits(o_bits)
