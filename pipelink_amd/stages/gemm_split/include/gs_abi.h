@@ -4,8 +4,8 @@
  *
  * The split follows the reference's three-package GEMM (examples/hopper-gemm-split: loader /
  * MMA / epilogue; contracts in src/channels.cuh:33-71) with GELU in place of its ReLU:
- *   gs.loader    role `load`, 1 wave: global -> LDS ring, one ring stage = 64 contraction
- *                elements of the tile's 128 A rows and 128 B rows (2 x 16 KB)
+ *   gs.loader    role `load`, 2 waves (one for the A rows, one for the B rows): global -> LDS ring, one ring
+ *                stage = 64 contraction elements of the tile's 128 A rows and 128 B rows (2 x 16 KB)
  *   gs.mma       role `mma`, 4 waves as 2 x 2, 64 x 64 outputs each: LDS -> MFMA 32x32x16 bf16
  *   gs.epilogue  an export the mma role calls with its accumulator: + bias, GELU, bf16 store */
 #ifndef PIPELINK_GS_ABI_H
@@ -18,6 +18,7 @@
 #define GS_TILE_N 128
 #define GS_TILE_K 64                    /* contraction elements per ring stage */
 #define GS_STAGE_BYTES (2 * 128 * 128)  /* A rows then B rows, 128 bytes each */
+#define GS_LOAD_WAVES 2                 /* arrivals on a stage's `full` counter per fill: one per loader wave */
 
 typedef struct GsLoaderParams {
   const uint16_t* a;  /* [M, K] bf16 */

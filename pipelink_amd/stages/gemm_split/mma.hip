@@ -2,8 +2,10 @@
 //
 // Four waves as 2 (rows) x 2 (columns), 64 x 64 outputs each = 2 x 2 accumulators of
 // v_mfma_f32_32x32x16_bf16.  Per ring stage (64 contraction elements) a wave waits for the
-// stage's `full` count, reads its two A fragments and two B fragments for each of the four
-// 16-element sub-steps from LDS, says on `empty` that it has read the stage, and multiplies.
+// stage's `full` count (one arrival per loader wave), reads its two A fragments and two B fragments for
+// each of the four 16-element sub-steps from LDS, half a stage at a time into one of two register sets (the
+// reads of one half are on their way while the other half is multiplied), and says on `empty` that it has
+// read the stage.
 // At the end it hands the accumulator to whoever serves the `epilogue` channel.
 //
 // MFMA 32x32x16 bf16 operand of lane l: row l % 32, contraction elements 8 * (l / 32) .. + 8 of
@@ -55,28 +57,42 @@ extern "C" __device__ void gs_mma_role_mma(const void* params, unsigned variant)
       for (int r = 0; r < 16; ++r) acc.v[i][j][r] = 0.0f;
   const int stages = p.k / GS_TILE_K;
   bool ok = true;
-  for (int s = 0; s < stages; ++s) {
+  // Fragment registers are double-buffered by half stages: while the 8 MFMAs of one half (two 16-element sub-steps)
+  // run, the 8 reads of the next half are on their way.  Set 0 holds a stage's first half, set 1 its second.
+  v8bf fa[2][2][2], fb[2][2][2];
+  auto read_half = [&](int s, int set) {
     const int slot = s % depth, use = s / depth;
-    ok &= pl::ring_wait(pl::ring_counter(pipelink_smem, pipelink_gs_full(), slot), (uint32_t)use + 1u);
+    if (set == 0) ok &= pl::ring_wait(pl::ring_counter(pipelink_smem, pipelink_gs_full(), slot), ((uint32_t)use + 1u) * GS_LOAD_WAVES);
     const unsigned char* a_rows = ring + slot * GS_STAGE_BYTES;
     const unsigned char* b_rows = a_rows + GS_TILE_M * 128;
-    v8bf a[4][2], b[4][2];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
+    for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        a[kk][i] = read_frag(a_rows, arow + 32 * i, 2 * kk + half);
-        b[kk][i] = read_frag(b_rows, brow + 32 * i, 2 * kk + half);
+        fa[set][k2][i] = read_frag(a_rows, arow + 32 * i, 2 * (2 * set + k2) + half);
+        fb[set][k2][i] = read_frag(b_rows, brow + 32 * i, 2 * (2 * set + k2) + half);
       }
-    pl::ring_wait_reads();
-    if (lane == 0) pl::ring_arrive(pl::ring_counter(pipelink_smem, pipelink_gs_empty(), slot));
+  };
+  auto multiply = [&](int set) {
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
+    for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc.v[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk][i], b[kk][j], acc.v[i][j], 0, 0, 0);
+        for (int j = 0; j < 2; ++j) acc.v[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][k2][i], fb[set][k2][j], acc.v[i][j], 0, 0, 0);
+  };
+  read_half(0, 0);
+  for (int s = 0; s < stages; ++s) {
+    read_half(s, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(0);
+    __builtin_amdgcn_sched_barrier(0);
+    pl::ring_wait_reads();  // both halves of stage s are in registers
+    if (lane == 0) pl::ring_arrive(pl::ring_counter(pipelink_smem, pipelink_gs_empty(), s % depth));
+    if (s + 1 < stages) read_half(s + 1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(1);
+    __builtin_amdgcn_sched_barrier(0);
   }
   if (!ok && lane == 0) atomicOr(p.status, 2u);
   const pipelink_host_view view{params, nullptr};
@@ -91,7 +107,7 @@ PL_PARAMS(GsMmaParams);
 PL_ROLE(mma, gs_mma_role_mma, 4);
 PL_TOPOLOGY(false, "static");
 PL_VARIANT(0, {});
-PL_RING(ab_ring, "consume", mma, "bf16", 16, 256, 64, "pipelink_gs_depth", 32768, "pipelink_gs_full", "1", load,
+PL_RING(ab_ring, "consume", mma, "bf16", 16, 256, 64, "pipelink_gs_depth", 32768, "pipelink_gs_full", "warps(load)", load,
         "pipelink_gs_empty", "warps(mma)", mma, load);
 PL_CLAIM_WARPS("pipelink_gs_warp_mma", mma, 4);
 PL_CALL(epilogue, "gs_epilogue_store",

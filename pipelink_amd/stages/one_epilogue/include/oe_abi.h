@@ -16,6 +16,7 @@
 #define OE_TILE 128
 #define OE_TILE_K 64
 #define OE_STAGE_BYTES (2 * 128 * 128)
+#define OE_LOAD_WAVES 2 /* the loader's waves: arrivals on a stage's `full` counter per fill (GS_LOAD_WAVES) */
 #define OE_LDS_PITCH (64 * 4 + 16) /* bytes between rows of a wave's 64 x 64 fp32 tile in LDS */
 
 typedef struct OeMmaParams {

@@ -16,7 +16,7 @@ PL_PARAMS(OeMmaParams);
 PL_ROLE(mma, oe_mma_agpr_role_mma, 4);
 PL_TOPOLOGY(false, "static");
 PL_VARIANT(0, {});
-PL_RING(ab_ring, "consume", mma, "bf16", 16, 256, 64, "pipelink_gs_depth", 32768, "pipelink_gs_full", "1", load,
+PL_RING(ab_ring, "consume", mma, "bf16", 16, 256, 64, "pipelink_gs_depth", 32768, "pipelink_gs_full", "warps(load)", load,
         "pipelink_gs_empty", "warps(mma)", mma, load);
 PL_CLAIM_WARPS("pipelink_oe_warp_mma", mma, 4);
 

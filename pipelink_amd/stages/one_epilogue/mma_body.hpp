@@ -45,27 +45,42 @@ __device__ __forceinline__ void role(const void* params, unsigned char* tile_lds
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
   const int stages = p.k / OE_TILE_K;
   bool ok = true;
-  for (int s = 0; s < stages; ++s) {
+  // Fragment registers are double-buffered by half stages: while the 8 MFMAs of one half (two 16-element sub-steps)
+  // run, the 8 reads of the next half are on their way.  Set 0 holds a stage's first half, set 1 its second.
+  v8bf fa[2][2][2], fb[2][2][2];
+  auto read_half = [&](int s, int set) {
     const int slot = s % depth, use = s / depth;
-    ok &= pl::ring_wait(pl::ring_counter(pipelink_smem, pipelink_gs_full(), slot), (uint32_t)use + 1u);
+    if (set == 0) ok &= pl::ring_wait(pl::ring_counter(pipelink_smem, pipelink_gs_full(), slot), ((uint32_t)use + 1u) * OE_LOAD_WAVES);
     const unsigned char* a_rows = ring + slot * OE_STAGE_BYTES;
     const unsigned char* b_rows = a_rows + OE_TILE * 128;
-    v8bf a[4][2], b[4][2];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
+    for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        a[kk][i] = read_frag(a_rows, arow + 32 * i, 2 * kk + half);
-        b[kk][i] = read_frag(b_rows, brow + 32 * i, 2 * kk + half);
+        fa[set][k2][i] = read_frag(a_rows, arow + 32 * i, 2 * (2 * set + k2) + half);
+        fb[set][k2][i] = read_frag(b_rows, brow + 32 * i, 2 * (2 * set + k2) + half);
       }
-    pl::ring_wait_reads();
-    if (lane == 0) pl::ring_arrive(pl::ring_counter(pipelink_smem, pipelink_gs_empty(), slot));
+  };
+  auto multiply = [&](int set) {
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
+    for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk][i], b[kk][j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][k2][i], fb[set][k2][j], acc[i][j], 0, 0, 0);
+  };
+  read_half(0, 0);
+  for (int s = 0; s < stages; ++s) {
+    read_half(s, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(0);
+    __builtin_amdgcn_sched_barrier(0);
+    pl::ring_wait_reads();  // both halves of stage s are in registers
+    if (lane == 0) pl::ring_arrive(pl::ring_counter(pipelink_smem, pipelink_gs_empty(), s % depth));
+    if (s + 1 < stages) read_half(s + 1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(1);
+    __builtin_amdgcn_sched_barrier(0);
   }
   if (!ok && lane == 0) atomicOr(p.status, 2u);
   const pipelink_host_view view{params, nullptr};

@@ -82,14 +82,14 @@ def test_link_records_three_packages_ring_depth_and_geometry(example):
     assert [e["stage_id"] for e in link["params"]["entries"]] == ["gs.loader", "gs.mma", "gs.epilogue"]
     assert [(e["offset"], e["bytes"]) for e in link["params"]["entries"]] == [(0, 40), (40, 16), (56, 24)]
     assert link["params"]["total_bytes"] == 80
-    assert link["threads"] == (4 + 1) * 64 == 320                       # four matrix waves + one loader wave
+    assert link["threads"] == (4 + 2) * 64 == 384                       # four matrix waves + two loader waves
     assert link["bindings"]["pipelink_gs_depth"] == [4, "solved"]        # deepest ring that fits 160 KB
     assert link["dyn_smem_bytes"] == 4 * 32768 + 2 * 4 * 16 == 131200   # ring + full/empty counter slots
-    assert link["bindings"]["pipelink_gs_warp_mma"][0] == 0
+    assert link["bindings"]["pipelink_gs_warp_load"][0] == 0 and link["bindings"]["pipelink_gs_warp_mma"][0] == 2
     exp = {e["channel"]: e for e in link["protocol_expansions"]}
     assert set(exp) == {"ab_ring", "epilogue"}
     ring = exp["ab_ring"]
-    assert (ring["kind"], ring["tx_full"], ring["arrive_full"], ring["arrive_empty"]) == ("mbarrier", 32768, 1, 4)
+    assert (ring["kind"], ring["tx_full"], ring["arrive_full"], ring["arrive_empty"]) == ("mbarrier", 32768, 2, 4)   # one arrival per loader wave, one per matrix wave
     assert ring["init_materializer"] == "dispatch" and ring["depth"] == "pipelink_gs_depth"
     assert exp["epilogue"]["kind"] == "call"
     obs = link["observed"]
@@ -273,7 +273,7 @@ def test_cli_launch_verb_runs_the_example(tmp_path):
     proc = subprocess.run(cmd, capture_output=True, text=True, cwd=ROOT, timeout=120)
     assert proc.returncode == 0, proc.stderr
     report = json.loads(proc.stdout)
-    assert report["geometry"] == {"grid": [16, 1, 1], "block": [320, 1, 1], "dynamic_smem_bytes": 131200}
+    assert report["geometry"] == {"grid": [16, 1, 1], "block": [384, 1, 1], "dynamic_smem_bytes": 131200}
     assert np.load(tmp_path / "status.npy")[0] == 0
     got = torch.from_numpy(np.load(tmp_path / "c.npy").view(np.int16)).view(torch.bfloat16).float().numpy()
     want = gg.gemm_bias_gelu_torch(a, b, bias).float().numpy()
