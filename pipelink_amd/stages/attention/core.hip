@@ -19,6 +19,7 @@
 #include <pipelink/stage.hpp>
 #ifndef PIPELINK_EMIT
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include "include/fa_abi.h"
 
 extern "C" __device__ int pipelink_fa_kv();  // byte offset of the K / V^T buffers in dynamic LDS
@@ -43,6 +44,7 @@ constexpr int BUF_BYTES = 2 * K_BYTES;
 typedef short v4s __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4s* lds_v4s;
 constexpr float MASKED = -1.0e30f;
+constexpr float RESCALE_SLACK = 8.0f;  // log2 units
 
 // Where the 16-byte chunk `chunk` of a key's row stands in its 256-byte LDS row.  K is read one key per lane, 16 lanes
 // = 16 consecutive keys at one chunk: the 16 rows must put that chunk in 16 different places.  V is read in columns,
@@ -123,37 +125,42 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
   const int li = lane & 15, dgroup = 16 * ((lane >> 4) & 1);  // position in the 16-lane group, the group's first d in a 32-row block
   // LDS addresses, kept few: a K fragment is at [key = 32 t + l32][chunk 2 kk + half] -> this lane's 8 places in
   // its row (the tile t is an immediate offset); a V column piece is at [key][chunk 4 db + c] -> 4 places per lane.
-  int k_at[8];
+  // (as pointers into both buffers of the pair: the loop adds nothing to them)
+  const unsigned char* k_at[2][8];
 #pragma unroll
-  for (int kk = 0; kk < 8; ++kk) k_at[kk] = l32 * (FA_D * 2) + 16 * k_place(l32, 2 * kk + half);
+  for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) k_at[pb][kk] = buf + pb * BUF_BYTES + l32 * (FA_D * 2) + 16 * k_place(l32, 2 * kk + half);
   const int v_key = 4 * half + (li >> 2);  // the key (within a group of 16) this lane points at for the transposing read
-  int v_at[4];
+  const unsigned char* v_at[2][4];
 #pragma unroll
-  for (int db = 0; db < 4; ++db) {
-    const int d = 32 * db + dgroup + 4 * (li & 3);
-    v_at[db] = v_key * (FA_D * 2) + 16 * v_place(v_key, d >> 3) + 2 * (d & 4);
-  }
+  for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+      const int d = 32 * db + dgroup + 4 * (li & 3);
+      v_at[pb][db] = buf + pb * BUF_BYTES + K_BYTES + v_key * (FA_D * 2) + 16 * v_place(v_key, d >> 3) + 2 * (d & 4);
+    }
   // the 8 pieces (4 blocks of d x two halves of 8 keys) of the group of 16 keys that starts at key `first`
-  auto read_v_group = [&](const unsigned char* vbuf, int first, v4s (&piece)[8]) {
+  auto read_v_group = [&](int pb, int first, v4s (&piece)[8]) {
 #pragma unroll
     for (int db = 0; db < 4; ++db) {
       // rows first + v_key and 8 further on: (key & 3) is the same, so is the place in the row
-      piece[2 * db] = read_v_piece(vbuf + v_at[db] + first * (FA_D * 2));
-      piece[2 * db + 1] = read_v_piece(vbuf + v_at[db] + (first + 8) * (FA_D * 2));
+      piece[2 * db] = read_v_piece(v_at[pb][db] + first * (FA_D * 2));
+      piece[2 * db + 1] = read_v_piece(v_at[pb][db] + (first + 8) * (FA_D * 2));
     }
   };
   issue_block<false>(kres, 0u, buf, wave, lane);
   issue_block<true>(vres, 0u, buf + K_BYTES, wave, lane);
-  for (int i = 0; i < blocks; ++i) {
-    unsigned char* kbuf = buf + (i & 1) * BUF_BYTES;
-    const unsigned char* vbuf = kbuf + K_BYTES;
+  // one block of 64 keys; PB = i % 2 (the buffer pair) is a compile-time constant so that the address tables are registers
+  auto block = [&](int i, auto pair) {
+    constexpr int PB = decltype(pair)::value;
     __syncthreads();  // blocks i of K and V have landed (the barrier drains every wave's loads); buffers of block i - 1 are free
     if (i + 1 < blocks) {
       issue_block<false>(kres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + ((i + 1) & 1) * BUF_BYTES, wave, lane);
       issue_block<true>(vres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + ((i + 1) & 1) * BUF_BYTES + K_BYTES, wave, lane);
     }
     const int k0 = i * FA_K_BLOCK;
-    if (k0 >= wave_keys) continue;  // no query of this wave sees a key this far on: only the loads and the barrier
+    if (k0 >= wave_keys) return;  // no query of this wave sees a key this far on: only the loads and the barrier
     // ---- S^T = K . Q^T : two 32-key tiles -----------------------------------------------------------
     v16f s[2];
     v4s piece[2][8];
@@ -162,7 +169,7 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk) kf[t][kk] = *reinterpret_cast<const v4i*>(kbuf + k_at[kk] + t * 32 * (FA_D * 2));
+        for (int kk = 0; kk < 8; ++kk) kf[t][kk] = *reinterpret_cast<const v4i*>(k_at[PB][kk] + t * 32 * (FA_D * 2));
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_setprio(2);
 #pragma unroll
@@ -172,7 +179,7 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, kf[t][kk]), qf[kk], s[t], 0, 0, 0);
       }
-      read_v_group(vbuf, 0, piece[0]);  // on their way during the softmax
+      read_v_group(PB, 0, piece[0]);  // on their way during the softmax
       __builtin_amdgcn_s_setprio(0);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -196,7 +203,12 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
     block_max = max_with_other_half(block_max);
     // every query sees key 0, and block 0 comes first: from then on the maximum is a real score, and a
     // masked entry (-1e30) turns into exp2(-huge) = 0 by itself
-    const float new_max = fmaxf(row_max, block_max * p.scale_log2e);
+    // The reference point of the exponentials only moves when a score exceeds it by more than 2^RESCALE_SLACK: until
+    // then probabilities may be as large as that (harmless in fp32 sums and bf16 operands, and the final division
+    // takes it out again), and the accumulated output and sum need no rescaling -- which they otherwise would
+    // in most blocks, because some query of the wave sees a new maximum.
+    const float top = block_max * p.scale_log2e;
+    const float new_max = top > row_max + RESCALE_SLACK ? top : row_max;
     const float alpha = __builtin_amdgcn_exp2f(row_max - new_max);
     row_max = new_max;
     float block_sum = 0.0f;
@@ -221,7 +233,7 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
 #pragma unroll
     for (int gi = 0; gi < 4; ++gi) {
       const int t = gi >> 1, g = gi & 1;
-      if (gi + 1 < 4) read_v_group(vbuf, 16 * (gi + 1), piece[(gi + 1) & 1]);
+      if (gi + 1 < 4) read_v_group(PB, 16 * (gi + 1), piece[(gi + 1) & 1]);
       __builtin_amdgcn_sched_barrier(0);
       v8f pf;
 #pragma unroll
@@ -236,6 +248,10 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
       __builtin_amdgcn_sched_barrier(0);
     }
     __builtin_amdgcn_s_setprio(0);
+  };
+  for (int i = 0; i < blocks; i += 2) {
+    block(i, std::integral_constant<int, 0>{});
+    if (i + 1 < blocks) block(i + 1, std::integral_constant<int, 1>{});
   }
   // ---- O[b][query][h][d] = O^T / row_sum, bf16 ------------------------------------------------------------
   const float inv = row_sum > 0.0f ? __builtin_amdgcn_rcpf(row_sum) : 0.0f;
