@@ -49,7 +49,7 @@ def test_link_records_core_and_mask_packages(example):
     assert link["threads"] == 256 and link["dyn_smem_bytes"] == 2 * 2 * 64 * 256 == 65536
     assert {e["channel"] for e in link["protocol_expansions"]} == {"mask_key_count", "mask_all_visible", "mask_visible"}
     obs = link["observed"]
-    assert obs["calls"] == 0 and obs["mfma"] == 32 and obs["private_segment_fixed_size"] == 0   # the mask is inlined
+    assert obs["calls"] == 0 and obs["mfma"] == 64 and obs["private_segment_fixed_size"] == 0   # the mask is inlined; the block loop is unrolled by two
     from pipelink_amd.stages.attention.params import params_blobs
     blobs = params_blobs({"q": 1, "k": 2, "v": 3, "o": 4}, 4, 32, 8, 4096)
     assert {sid: len(b) for sid, b in blobs.items()} == {"fa.core": 56, "fa.mask.causal": 8}
