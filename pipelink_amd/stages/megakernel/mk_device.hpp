@@ -57,7 +57,7 @@ __device__ __forceinline__ void my_rows(int total, int& first, int& last) {
 
 // Lane exchanges inside a row of 16 lanes as DPP operands of the add itself (no LDS round trip as a shuffle is):
 // 0xB1 / 0x4E swap neighbours / pairs inside a quad, 0x141 mirrors each half row (swaps its quads), 0x140 mirrors
-// the row (swaps its halves), 0x104 reads the lane four further on, 0x128 the lane eight away.
+// the row (swaps its halves), 0x104 / 0x108 read the lane four / eight further on, 0x128 the lane eight away (rotating).
 template <int CTRL>
 __device__ __forceinline__ float dpp(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
