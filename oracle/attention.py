@@ -24,12 +24,16 @@ def inputs(batch: int, q_heads: int, kv_heads: int, seq: int, dim: int = 128, se
     return q, k, v
 
 
-def attention_head(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float | None = None) -> torch.Tensor:
-    """One head: q, k, v [S, D] -> [S, D] fp32, causal."""
+def attention_head(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float | None = None, window: int | None = None) -> torch.Tensor:
+    """One head: q, k, v [S, D] -> [S, D] fp32, causal; with `window`, a query sees only the last `window` keys up to
+    its own (campaigns/attention/src/sm90/stage_mask_window.cu: kv_pos > q_pos - window)."""
     s, d = q.shape
     scale = 1.0 / math.sqrt(d) if scale is None else scale
     scores = (q.float() @ k.float().t()) * scale
-    scores = scores.masked_fill(torch.ones(s, s, dtype=torch.bool).triu(1), float("-inf"))
+    hidden = torch.ones(s, s, dtype=torch.bool).triu(1)
+    if window is not None:
+        hidden |= torch.ones(s, s, dtype=torch.bool).tril(-window)
+    scores = scores.masked_fill(hidden, float("-inf"))
     return torch.softmax(scores, dim=-1) @ v.float()
 
 
@@ -37,9 +41,10 @@ def attention_head_library(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) ->
     return torch.nn.functional.scaled_dot_product_attention(q.float()[None], k.float()[None], v.float()[None], is_causal=True)[0]
 
 
-def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: list[tuple[int, int]] | None = None) -> dict[tuple[int, int], torch.Tensor]:
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: list[tuple[int, int]] | None = None,
+              window: int | None = None) -> dict[tuple[int, int], torch.Tensor]:
     """{(batch, query head): [S, D] fp32} for the listed heads (all if None)."""
     b, hq, _, _ = q.shape
     group = hq // k.shape[1]
     heads = [(i, h) for i in range(b) for h in range(hq)] if heads is None else heads
-    return {(i, h): attention_head(q[i, h], k[i, h // group], v[i, h // group]) for i, h in heads}
+    return {(i, h): attention_head(q[i, h], k[i, h // group], v[i, h // group], window=window) for i, h in heads}

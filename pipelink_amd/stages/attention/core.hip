@@ -24,6 +24,7 @@
 
 extern "C" __device__ int pipelink_fa_kv();  // byte offset of the K / V^T buffers in dynamic LDS
 extern "C" __device__ int pipelink_call_mask_key_count(const void* view, int q_first, int q_last);
+extern "C" __device__ int pipelink_call_mask_key_begin(const void* view, int q_first, int q_last);
 extern "C" __device__ int pipelink_call_mask_all_visible(const void* view, int q_first, int q_last, int k_first, int k_last);
 extern "C" __device__ int pipelink_call_mask_visible(const void* view, int q, int k);
 
@@ -115,9 +116,11 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
     for (int r = 0; r < 16; ++r) o[db][r] = 0.0f;
   float row_max = MASKED, row_sum = 0.0f;
 
+  // the mask package says which stretch of keys the tile's queries may see at all: blocks [first_block, blocks)
   const int keys = pipelink_call_mask_key_count(&view, q0, q0 + FA_Q_TILE - 1);
+  const int first_block = pipelink_call_mask_key_begin(&view, q0, q0 + FA_Q_TILE - 1) / FA_K_BLOCK;
   const int blocks = (keys + FA_K_BLOCK - 1) / FA_K_BLOCK;
-  const int wave_keys = pipelink_call_mask_key_count(&view, qw, qw + 31);
+  const int wave_keys = pipelink_call_mask_key_count(&view, qw, qw + 31), wave_begin = pipelink_call_mask_key_begin(&view, qw, qw + 31);
   // Schedule.  Two LDS buffers per operand: block i + 1 is in flight while block i is multiplied; one barrier per
   // block.  LDS reads are issued in batches ahead of the MFMAs that use them (a read costs a few hundred clocks of
   // latency, an MFMA 32): all 16 K fragments of a block before its first score MFMA, the V pieces of the next group
@@ -149,18 +152,18 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
       piece[2 * db + 1] = read_v_piece(v_at[pb][db] + (first + 8) * (FA_D * 2));
     }
   };
-  issue_block<false>(kres, 0u, buf, wave, lane);
-  issue_block<true>(vres, 0u, buf + K_BYTES, wave, lane);
-  // one block of 64 keys; PB = i % 2 (the buffer pair) is a compile-time constant so that the address tables are registers
+  issue_block<false>(kres, (uint32_t)first_block * FA_K_BLOCK * FA_D * 2, buf, wave, lane);
+  issue_block<true>(vres, (uint32_t)first_block * FA_K_BLOCK * FA_D * 2, buf + K_BYTES, wave, lane);
+  // one block of 64 keys; PB = (i - first_block) % 2 (the buffer pair) is a compile-time constant so that the address tables are registers
   auto block = [&](int i, auto pair) {
     constexpr int PB = decltype(pair)::value;
     __syncthreads();  // blocks i of K and V have landed (the barrier drains every wave's loads); buffers of block i - 1 are free
     if (i + 1 < blocks) {
-      issue_block<false>(kres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + ((i + 1) & 1) * BUF_BYTES, wave, lane);
-      issue_block<true>(vres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + ((i + 1) & 1) * BUF_BYTES + K_BYTES, wave, lane);
+      issue_block<false>(kres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + (1 - PB) * BUF_BYTES, wave, lane);
+      issue_block<true>(vres, (uint32_t)(i + 1) * FA_K_BLOCK * FA_D * 2, buf + (1 - PB) * BUF_BYTES + K_BYTES, wave, lane);
     }
     const int k0 = i * FA_K_BLOCK;
-    if (k0 >= wave_keys) return;  // no query of this wave sees a key this far on: only the loads and the barrier
+    if (k0 >= wave_keys || k0 + FA_K_BLOCK <= wave_begin) return;  // no query of this wave sees a key of this block: only the loads and the barrier
     // ---- S^T = K . Q^T : two 32-key tiles -----------------------------------------------------------
     v16f s[2];
     v4s piece[2][8];
@@ -201,8 +204,8 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
 #pragma unroll
       for (int r = 0; r < 16; ++r) block_max = fmaxf(block_max, s[t][r]);
     block_max = max_with_other_half(block_max);
-    // every query sees key 0, and block 0 comes first: from then on the maximum is a real score, and a
-    // masked entry (-1e30) turns into exp2(-huge) = 0 by itself
+    // once a query has seen a key its maximum is a real score, and a masked entry (-1e30) turns into exp2(-huge) = 0
+    // by itself
     // The reference point of the exponentials only moves when a score exceeds it by more than 2^RESCALE_SLACK: until
     // then probabilities may be as large as that (harmless in fp32 sums and bf16 operands, and the final division
     // takes it out again), and the accumulated output and sum need no rescaling -- which they otherwise would
@@ -211,12 +214,15 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
     const float new_max = top > row_max + RESCALE_SLACK ? top : row_max;
     const float alpha = __builtin_amdgcn_exp2f(row_max - new_max);
     row_max = new_max;
+    // a query that has not seen a key yet (a window mask: the block's keys are all too old for it) has no real maximum
+    // to lean on: its exponentials are taken against +huge instead, which makes every one of them 0
+    const float reference = new_max < 0.01f * MASKED ? -MASKED : new_max;
     float block_sum = 0.0f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], p.scale_log2e, -new_max));
+        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], p.scale_log2e, -reference));
         s[t][r] = e;
         block_sum += e;
       }
@@ -249,7 +255,7 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
     }
     __builtin_amdgcn_s_setprio(0);
   };
-  for (int i = 0; i < blocks; i += 2) {
+  for (int i = first_block; i < blocks; i += 2) {
     block(i, std::integral_constant<int, 0>{});
     if (i + 1 < blocks) block(i + 1, std::integral_constant<int, 1>{});
   }
@@ -276,6 +282,8 @@ PL_TOPOLOGY(false, "static");
 PL_VARIANT(0, {});
 PL_CALL(mask_key_count, "mask_key_count",
         "extern \"C\" __device__ int pipelink_call_mask_key_count(const void* view, int q_first, int q_last);");
+PL_CALL(mask_key_begin, "mask_key_begin",
+        "extern \"C\" __device__ int pipelink_call_mask_key_begin(const void* view, int q_first, int q_last);");
 PL_CALL(mask_all_visible, "mask_all_visible",
         "extern \"C\" __device__ int pipelink_call_mask_all_visible(const void* view, int q_first, int q_last, int k_first, int k_last);");
 PL_CALL(mask_visible, "mask_visible",

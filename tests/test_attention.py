@@ -32,6 +32,15 @@ def test_oracle_against_the_library_and_closed_forms():
     assert torch.allclose(mean, running, rtol=1e-5, atol=1e-6)              # equal scores: a running mean of V
     heads = oa.attention(q, k, v)
     assert set(heads) == {(0, 0), (0, 1)} and torch.equal(heads[(0, 1)], mine)   # both query heads read KV head 0
+    # sliding window: one key -> the query's own V row; a window as long as the sequence -> plain causal; equal
+    # scores -> the mean of the last `window` rows of V
+    assert torch.allclose(oa.attention_head(q[0, 1], k[0, 0], v[0, 0], window=1), v[0, 0].float())
+    assert torch.equal(oa.attention_head(q[0, 1], k[0, 0], v[0, 0], window=96), mine)
+    vf = v[0, 0].float()
+    sums = vf.cumsum(0)
+    sums[5:] -= vf.cumsum(0)[:-5].clone()
+    last5 = sums / torch.arange(1, 97).clamp(max=5)[:, None]
+    assert torch.allclose(oa.attention_head(q[0, 0], same_k, v[0, 0], window=5), last5, rtol=1e-4, atol=1e-5)
 
 
 @pytest.fixture(scope="module")
@@ -47,12 +56,25 @@ def test_link_records_core_and_mask_packages(example):
     assert [e["stage_id"] for e in link["params"]["entries"]] == ["fa.core", "fa.mask.causal"]
     assert [(e["offset"], e["bytes"]) for e in link["params"]["entries"]] == [(0, 56), (56, 8)]
     assert link["threads"] == 256 and link["dyn_smem_bytes"] == 2 * 2 * 64 * 256 == 65536
-    assert {e["channel"] for e in link["protocol_expansions"]} == {"mask_key_count", "mask_all_visible", "mask_visible"}
+    assert {e["channel"] for e in link["protocol_expansions"]} == {"mask_key_count", "mask_key_begin", "mask_all_visible", "mask_visible"}
     obs = link["observed"]
     assert obs["calls"] == 0 and obs["mfma"] == 64 and obs["private_segment_fixed_size"] == 0   # the mask is inlined; the block loop is unrolled by two
     from pipelink_amd.stages.attention.params import params_blobs
     blobs = params_blobs({"q": 1, "k": 2, "v": 3, "o": 4}, 4, 32, 8, 4096)
     assert {sid: len(b) for sid, b in blobs.items()} == {"fa.core": 56, "fa.mask.causal": 8}
+
+
+@needs_rocm
+def test_window_mask_is_a_relink_of_the_same_core_package(example):
+    out, res = example
+    link, window = res["link"], res["window"]
+    assert [e["stage_id"] for e in window["params"]["entries"]] == ["fa.core", "fa.mask.window"]
+    assert window["input_hashes"]["fa.core"] == link["input_hashes"]["fa.core"]   # the same package bytes went into both links
+    assert set(window["input_hashes"]) == {"fa.core", "fa.mask.window"}
+    assert window["observed"]["calls"] == 0 and window["observed"]["mfma"] == 64
+    from pipelink_amd.stages.attention.params import params_blobs
+    blobs = params_blobs({"q": 1, "k": 2, "v": 3, "o": 4}, 4, 32, 8, 4096, window=1024)
+    assert set(blobs) == {"fa.core", "fa.mask.window"} and blobs["fa.mask.window"] == (4096).to_bytes(4, "little") + (1024).to_bytes(4, "little")
 
 
 def test_host_rejects_shapes_the_kernel_does_not_handle():
@@ -100,6 +122,31 @@ def test_small_case_matches_the_oracle_on_every_head():
     finally:
         sess.close()
     _check_heads(o, q, k, v, None)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("window", [1, 100, 128, 300, 4096])
+def test_window_mask_matches_the_oracle_on_every_head(window):
+    """The relinked image (fa.core + fa.mask.window): windows below, at and above the 64-key block and the 128-query
+    tile, and one longer than the sequence (plain causal)."""
+    from pipelink_amd.host.attention import open_session
+
+    paths = fa_build.images()
+    q, k, v = oa.inputs(1, 4, 2, 640, seed=5)
+    sess = open_session(paths["window_link_json"], _bits(q), _bits(k), _bits(v), window=window)
+    try:
+        sess.write("o", np.full((1, 640, 512), 0x7FC0, dtype=np.uint16))
+        sess.launch()
+        sess.synchronize()
+        o = _from_bits(sess.read("o"))
+    finally:
+        sess.close()
+    ref = oa.attention(q, k, v, None, window=window)
+    for (b, h), want in ref.items():
+        got = o[b, :, h * 128:(h + 1) * 128]
+        assert torch.isfinite(got).all()
+        assert (got - want).abs().max().item() <= 1e-2 * want.abs().max().item(), (b, h)
+        assert ((got - want).norm() / want.norm()).item() <= 1e-2, (b, h)
 
 
 @pytest.mark.gpu
