@@ -97,16 +97,28 @@ def open_hostless(link_json: str | Path | dict, *, buffers: dict[str, Any], para
         backend = HipBackend(device)
     backend.current()
     placed: dict[str, tuple[int, int, Any]] = {}
+    owned: list[int] = []   # device allocations of this call: given back if the session cannot be opened
+    try:
+        return _open_placed(link, base, buffers, params, grid, backend, image, placed, owned)
+    except BaseException:
+        for addr in owned:
+            backend.free(addr)
+        raise
+
+
+def _open_placed(link, base, buffers, params, grid, backend, image, placed, owned) -> HostlessSession:
     for name, spec in buffers.items():
         if isinstance(spec, np.ndarray):
             data = np.ascontiguousarray(spec)
             addr = backend.allocate(max(data.nbytes, 1))
+            owned.append(addr)
             backend.upload(addr, data.tobytes())
             placed[name] = (addr, data.nbytes, (data.shape, data.dtype))
         else:
             shape, dtype = spec
             size = int(np.prod(shape)) * np.dtype(dtype).itemsize
             addr = backend.allocate(max(size, 1))
+            owned.append(addr)
             backend.zero(addr, size)
             placed[name] = (addr, size, (tuple(shape), np.dtype(dtype)))
     backend.synchronize()
@@ -123,6 +135,7 @@ def open_hostless(link_json: str | Path | dict, *, buffers: dict[str, Any], para
                   expected=e["bytes"], actual=len(blob))
         image_bytes[e["offset"]:e["offset"] + e["bytes"]] = blob
     params_addr = backend.allocate(len(image_bytes))
+    owned.append(params_addr)
     backend.upload(params_addr, bytes(image_bytes))
     path = Path(image) if image else base / link["target"]["image"]
     module = backend.module_load(path.read_bytes())

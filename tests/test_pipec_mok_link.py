@@ -190,9 +190,12 @@ def test_hostless_launcher_params_contract(cell):
     other.launch()
     assert len(be.launches) == 2 and be.launches[1][0] == s.params_addr   # shared params and buffers
     s.close()
+    refused = MemoryBackend()
     with pytest.raises(LaunchError) as err:
-        open_hostless(link, buffers={}, params=lambda a: {"mok.gemm": b"\0" * 264}, grid=(1,), backend=MemoryBackend(), image=image)
+        open_hostless(link, buffers={"a": np.arange(4, dtype=np.int32)}, params=lambda a: {"mok.gemm": b"\0" * 264}, grid=(1,),
+                      backend=refused, image=image)
     assert err.value.clause_ids == {"L-PARAMS"} and err.value.failures[0].path == "launch.params"
+    assert refused.log.count("allocate") == 1 and not refused.mem       # a refused open gives its device memory back
     with pytest.raises(LaunchError):
         open_hostless(link, buffers={}, params=lambda a: {"mok.framework": b"", "mok.gemm": b"", "mok.act": b""}, grid=(1,),
                       backend=MemoryBackend(), image=image)
