@@ -5,7 +5,8 @@
  * Packages (campaigns/megakernel/port/src in the reference: interpreter.cu + ops/*.cu wrapped as opcode
  * slots): mk.interp -- the persistent role: every workgroup walks the same instruction stream, calls the
  * op an instruction names through a call channel with its share of the work, and meets the others at a
- * grid barrier where an instruction asks for one -- and eight op packages: mk.rmsnorm, mk.qkv, mk.rope,
+ * grid barrier where an instruction asks for one (arriving after the op, waiting inside the next one: MkPending
+ * below) -- and eight op packages: mk.rmsnorm, mk.qkv, mk.rope,
  * mk.attn, mk.oproj, mk.upgate, mk.down, mk.lmhead.  Swapping the attention package (mk.attn for
  * mk.attn.wide) and relinking changes nothing else.
  *
@@ -39,6 +40,18 @@
 typedef struct MkInstr {
   int32_t opcode, layer, barrier_after, reserved;
 } MkInstr;
+
+/* What stands between an op and its inputs when the interpreter calls it.  A grid barrier is in two halves: a
+ * workgroup arrives when it has finished an op, and waits for the others only when the next op needs what they
+ * wrote.  An op therefore first asks for what depends on nobody -- its first rows of weights, its first stretch of
+ * the cache -- and then calls the interpreter's `op_inputs` channel once, which waits for the barrier (if one is
+ * open) and runs the normalisation that fills the workgroup's LDS vector (if the instruction before was one).
+ * Before that call an op may read only what no op writes during the step and may not touch the LDS vector.  An op
+ * that returns without the call has the interpreter make it. */
+typedef struct MkPending {
+  const MkInstr* norm; /* an rmsnorm instruction whose result the op needs, or null */
+  uint32_t barrier;    /* the barrier generation to wait for, 0: none */
+} MkPending;
 
 typedef struct MkModel {
   const uint16_t* weights; /* bf16; per layer: attn_norm[D], wqkv[(HQ+2HKV)*64][D], wo[D][HQ*64], ffn_norm[D], wgate[DFF][D],

@@ -4,6 +4,10 @@
 // (MkModel.program); an instruction names an op, the op's package does this workgroup's share of it.
 // Where an instruction asks for it, the workgroups meet at a grid barrier: a counter in global memory
 // that only grows, so that what one workgroup wrote (on any XCD) before it is what the others read after it.
+// The barrier is in two halves.  A workgroup arrives as soon as its op is done and goes on into the next op, which
+// first asks memory for what no workgroup writes (its first rows of weights, its stretch of the cache) and only
+// then calls back (channel inputs_<op>) to wait for the others: the barrier's 2.5 us and the first loads' latency
+// run side by side.  A normalisation instruction is held back in the same way and runs inside that call.
 // The wait is a bounded poll: a workgroup that gives up raises the status word and goes on, it never
 // spins for ever.
 #include <pipelink/stage.hpp>
@@ -11,12 +15,12 @@
 #include "mk_device.hpp"
 
 extern "C" __device__ void pipelink_call_op_rmsnorm(const void* view, const MkInstr* instr);
-extern "C" __device__ void pipelink_call_op_qkv(const void* view, const MkInstr* instr);
-extern "C" __device__ void pipelink_call_op_attn(const void* view, const MkInstr* instr);
-extern "C" __device__ void pipelink_call_op_oproj(const void* view, const MkInstr* instr);
-extern "C" __device__ void pipelink_call_op_upgate(const void* view, const MkInstr* instr);
-extern "C" __device__ void pipelink_call_op_down(const void* view, const MkInstr* instr);
-extern "C" __device__ void pipelink_call_op_lmhead(const void* view, const MkInstr* instr);
+extern "C" __device__ void pipelink_call_op_qkv(const void* view, const MkInstr* instr, MkPending* pending);
+extern "C" __device__ void pipelink_call_op_attn(const void* view, const MkInstr* instr, MkPending* pending);
+extern "C" __device__ void pipelink_call_op_oproj(const void* view, const MkInstr* instr, MkPending* pending);
+extern "C" __device__ void pipelink_call_op_upgate(const void* view, const MkInstr* instr, MkPending* pending);
+extern "C" __device__ void pipelink_call_op_down(const void* view, const MkInstr* instr, MkPending* pending);
+extern "C" __device__ void pipelink_call_op_lmhead(const void* view, const MkInstr* instr, MkPending* pending);
 
 // the opcode numbers the link bound to the op packages' claims
 extern "C" __device__ int pipelink_mk_opcode_rmsnorm_attn();
@@ -60,46 +64,90 @@ __device__ __forceinline__ bool poll(uint32_t* word, uint32_t target, bool local
   __hip_atomic_fetch_or(m.sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return false;
 }
-__device__ __forceinline__ void grid_barrier(const MkModel& m, uint32_t& passed) {
+// first half of barrier number `generation` (1, 2, ...): this workgroup has finished what comes before it
+__device__ __forceinline__ void grid_arrive(const MkModel& m, uint32_t generation) {
   __syncthreads();  // every wave's stores have been issued and acknowledged by the L2
-  ++passed;
   if (threadIdx.x == 0) {
     const uint32_t xcd = blockIdx.x % NUM_XCD;
-    const uint32_t members = (gridDim.x - xcd + NUM_XCD - 1) / NUM_XCD, groups = min((uint32_t)NUM_XCD, gridDim.x);
-    uint32_t* mine = m.sync + XCD_COUNTER * (1 + xcd);
-    const uint32_t before = __hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (before + 1 == passed * members)
+    const uint32_t members = (gridDim.x - xcd + NUM_XCD - 1) / NUM_XCD;
+    const uint32_t before = __hip_atomic_fetch_add(m.sync + XCD_COUNTER * (1 + xcd), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (before + 1 == generation * members)
       __hip_atomic_fetch_add(m.sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+// second half: every workgroup has arrived at barrier number `generation`
+__device__ __forceinline__ void grid_wait(const MkModel& m, uint32_t generation) {
+  if (threadIdx.x == 0) {
+    const uint32_t xcd = blockIdx.x % NUM_XCD, groups = min((uint32_t)NUM_XCD, gridDim.x);
+    uint32_t* mine = m.sync + XCD_COUNTER * (1 + xcd);
     if (blockIdx.x < NUM_XCD) {  // this XCD's first workgroup listens for the grid
-      poll(m.sync, passed * groups, false, m);
-      __hip_atomic_exchange(mine + 1, passed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      poll(m.sync, generation * groups, false, m);
+      __hip_atomic_exchange(mine + 1, generation, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     } else {
-      poll(mine + 1, passed, true, m);
+      poll(mine + 1, generation, true, m);
     }
   }
   __syncthreads();
 }
 }  // namespace mk_interp
 
+// The ops' way to their inputs: the open barrier, then the normalisation that is due.
+__device__ __forceinline__ void mk_interp_inputs(const void* view, MkPending* pending) {
+  const MkModel& m = *static_cast<const MkModel*>(static_cast<const pipelink_host_view*>(view)->residue);
+  if (pending->barrier != 0) {
+    mk_interp::grid_wait(m, pending->barrier);
+    pending->barrier = 0;
+  }
+  if (pending->norm != nullptr) {
+    pipelink_call_op_rmsnorm(view, pending->norm);
+    pending->norm = nullptr;
+    __syncthreads();  // the op reads what the normalisation left in LDS
+  }
+}
+
+// a channel has one caller: one export per op package
+#define MK_INPUTS(name) \
+  extern "C" __device__ void mk_interp_inputs_##name(const void* view, MkPending* pending) { mk_interp_inputs(view, pending); }
+MK_INPUTS(qkv)
+MK_INPUTS(attn)
+MK_INPUTS(oproj)
+MK_INPUTS(upgate)
+MK_INPUTS(down)
+MK_INPUTS(lmhead)
+#undef MK_INPUTS
+
 extern "C" __device__ void mk_interp_role_worker(const void* params, unsigned variant) {
   (void)variant;
   const MkModel& m = *static_cast<const MkModel*>(params);
   const pipelink_host_view view{params, nullptr};
   uint32_t passed = 0;
+  MkPending pending{nullptr, 0};
   for (int i = 0; i < m.num_instr; ++i) {
     const MkInstr* instr = m.program + i;
     const int op = instr->opcode;  // uniform over the grid; the numbers are bound at link time
-    if (op == pipelink_mk_opcode_rmsnorm_attn() || op == pipelink_mk_opcode_rmsnorm_ffn() || op == pipelink_mk_opcode_rmsnorm_final())
+    const bool norm = op == pipelink_mk_opcode_rmsnorm_attn() || op == pipelink_mk_opcode_rmsnorm_ffn() || op == pipelink_mk_opcode_rmsnorm_final();
+    if (norm && pending.norm == nullptr && !instr->barrier_after) {
+      pending.norm = instr;  // runs when the next op asks for its inputs: that op's first loads are on their way by then
+      continue;
+    }
+    if (norm) {
+      mk_interp_inputs(&view, &pending);
       pipelink_call_op_rmsnorm(&view, instr);
-    else if (op == pipelink_mk_opcode_qkv()) pipelink_call_op_qkv(&view, instr);
-    else if (op == pipelink_mk_opcode_attn()) pipelink_call_op_attn(&view, instr);
-    else if (op == pipelink_mk_opcode_oproj()) pipelink_call_op_oproj(&view, instr);
-    else if (op == pipelink_mk_opcode_upgate()) pipelink_call_op_upgate(&view, instr);
-    else if (op == pipelink_mk_opcode_down()) pipelink_call_op_down(&view, instr);
-    else if (op == pipelink_mk_opcode_lmhead()) pipelink_call_op_lmhead(&view, instr);
-    if (instr->barrier_after) mk_interp::grid_barrier(m, passed);
-    else __syncthreads();  // the next op of this workgroup reads what this one left in LDS
+    } else if (op == pipelink_mk_opcode_qkv()) pipelink_call_op_qkv(&view, instr, &pending);
+    else if (op == pipelink_mk_opcode_attn()) pipelink_call_op_attn(&view, instr, &pending);
+    else if (op == pipelink_mk_opcode_oproj()) pipelink_call_op_oproj(&view, instr, &pending);
+    else if (op == pipelink_mk_opcode_upgate()) pipelink_call_op_upgate(&view, instr, &pending);
+    else if (op == pipelink_mk_opcode_down()) pipelink_call_op_down(&view, instr, &pending);
+    else if (op == pipelink_mk_opcode_lmhead()) pipelink_call_op_lmhead(&view, instr, &pending);
+    mk_interp_inputs(&view, &pending);  // an opcode nobody claimed, or an op that had nothing to do
+    if (instr->barrier_after) {
+      mk_interp::grid_arrive(m, ++passed);
+      pending.barrier = passed;
+    } else {
+      __syncthreads();  // the next op of this workgroup reads what this one left in LDS
+    }
   }
+  mk_interp_inputs(&view, &pending);
   // The last workgroup to get here puts the barrier counter back to zero for the next launch: by then every
   // workgroup has left its last barrier.
   if (threadIdx.x == 0) {
@@ -123,14 +171,25 @@ PL_PARAMS(MkModel);
 PL_ROLE(worker, mk_interp_role_worker, 4);
 PL_TOPOLOGY(true, "static");
 PL_VARIANT(0, {});
-#define MK_CALL(name) PL_CALL(op_##name, "op_" #name, "extern \"C\" __device__ void pipelink_call_op_" #name "(const void* view, const MkInstr* instr);")
-MK_CALL(rmsnorm);
+PL_CALL(op_rmsnorm, "op_rmsnorm", "extern \"C\" __device__ void pipelink_call_op_rmsnorm(const void* view, const MkInstr* instr);");
+#define MK_CALL(name) \
+  PL_CALL(op_##name, "op_" #name, "extern \"C\" __device__ void pipelink_call_op_" #name "(const void* view, const MkInstr* instr, MkPending* pending);")
 MK_CALL(qkv);
 MK_CALL(attn);
 MK_CALL(oproj);
 MK_CALL(upgate);
 MK_CALL(down);
 MK_CALL(lmhead);
+// what an op calls once before it reads its inputs (MkPending in include/mk_abi.h)
+#define MK_SERVE_INPUTS(name)                                                                                                      \
+  PL_EXPORT(inputs_##name, mk_interp_inputs_##name, "extern \"C\" __device__ void mk_interp_inputs_" #name "(const void* view, MkPending* pending);"); \
+  PL_SERVE(inputs_##name, "inputs_" #name)
+MK_SERVE_INPUTS(qkv);
+MK_SERVE_INPUTS(attn);
+MK_SERVE_INPUTS(oproj);
+MK_SERVE_INPUTS(upgate);
+MK_SERVE_INPUTS(down);
+MK_SERVE_INPUTS(lmhead);
 // the workgroup's activation vector: the normalised residual (D floats), the attention output (HQ * 64) or
 // the FFN intermediate (DFF floats), whichever the running op needs; 32 KB holds DFF = 8192, and 1 KB behind it is
 // the ops' reduction scratch

@@ -148,8 +148,10 @@ __device__ __forceinline__ void rows_dot(const uint16_t* rows, int64_t pitch, co
 
 // y(row) for this workgroup's rows [first, last) of a matrix with rows of n elements: waves take groups of R rows.
 // Rows of up to 2048 elements are one pass each, and then a wave loads its next group before it sums the present one.
-template <int R, typename Emit>
-__device__ __forceinline__ void matvec(const uint16_t* w, int n, const float* x, int first, int last, Emit&& emit) {
+// `ready` is called once, by every thread, after the wave's first loads have been issued and before x is read:
+// the place to wait for x.
+template <int R, typename Emit, typename Ready>
+__device__ __forceinline__ void matvec(const uint16_t* w, int n, const float* x, int first, int last, Emit&& emit, Ready&& ready) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int r = first + R * wave;
   auto finish = [&](const v4i (&loaded)[R][4], int row) {
@@ -163,6 +165,7 @@ __device__ __forceinline__ void matvec(const uint16_t* w, int n, const float* x,
   if (r + R <= last) {
     v4i wa[R][4], wb[R][4];
     rows_load<R>(w + (int64_t)r * n, n, n, lane, wa);
+    ready();
     for (;;) {
       int next = r + 4 * R;
       bool more = next + R <= last;
@@ -177,6 +180,8 @@ __device__ __forceinline__ void matvec(const uint16_t* w, int n, const float* x,
       r = next;
       if (!more) break;
     }
+  } else {
+    ready();
   }
   for (; r < last; ++r) {  // a last group with fewer than R rows
     float sum[1];
@@ -192,6 +197,10 @@ template <int R>
 __device__ __forceinline__ void split_load(const uint16_t* rows, int n, v4i (&w)[R][4]) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   rows_load<R>(rows + wave * (n / 4), n, n / 4, lane, w);
+}
+template <int R, typename Emit>
+__device__ __forceinline__ void matvec(const uint16_t* w, int n, const float* x, int first, int last, Emit&& emit) {
+  matvec<R>(w, n, x, first, last, emit, [] {});
 }
 template <int R, typename Emit>
 __device__ __forceinline__ void matvec_split(const uint16_t* rows, int n, const float* x, float* scratch, int count, const v4i (&loaded)[R][4], Emit&& emit) {

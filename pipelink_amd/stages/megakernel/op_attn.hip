@@ -6,6 +6,7 @@
 #include "mk_device.hpp"
 
 extern "C" __device__ float pipelink_call_rope_apply(const void* view, const float* v, int i);
+extern "C" __device__ void pipelink_call_inputs_attn(const void* view, MkPending* pending);
 
 namespace mk_attn {
 __device__ __forceinline__ float bf16_round(float x) {
@@ -15,7 +16,7 @@ __device__ __forceinline__ float bf16_round(float x) {
 }
 }  // namespace mk_attn
 
-extern "C" __device__ void mk_attn_op(const void* view, const MkInstr* instr) {
+extern "C" __device__ void mk_attn_op(const void* view, const MkInstr* instr, MkPending* pending) {
   const MkModel& m = mk::model(view);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int head = blockIdx.x / m.chunks, chunk = blockIdx.x % m.chunks;
@@ -45,6 +46,7 @@ extern "C" __device__ void mk_attn_op(const void* view, const MkInstr* instr) {
   for (int j = 0; j < AHEAD; ++j) kreg[j] = *reinterpret_cast<const mk::v4i*>(kc + min(pl0 + 32 * j, last_cached) * pos_stride + 8 * piece);
 #pragma unroll
   for (int j = 0; j < AHEAD; ++j) vreg[j] = *reinterpret_cast<const mk::v4i*>(vc + min(pl0 + 32 * j, last_cached) * pos_stride + 8 * piece);
+  pipelink_call_inputs_attn(view, pending);  // the cache reads above depend on nobody; the query, key and value of this step do
   if (tid < 64) q[tid] = pipelink_call_rope_apply(view, m.qkv + head * MK_HEAD_DIM, tid);
   else if (tid < 128) knew[tid - 64] = mk_attn::bf16_round(pipelink_call_rope_apply(view, m.qkv + (m.hq + kvh) * MK_HEAD_DIM, tid - 64));
   __syncthreads();
@@ -147,7 +149,8 @@ PL_STAGE("mk.attn", "0.1.0");
 PL_NO_PARAMS();
 PL_TOPOLOGY(true, "static");
 PL_VARIANT(0, {});
-PL_EXPORT(op_attn, mk_attn_op, "extern \"C\" __device__ void mk_attn_op(const void* view, const MkInstr* instr);");
+PL_EXPORT(op_attn, mk_attn_op, "extern \"C\" __device__ void mk_attn_op(const void* view, const MkInstr* instr, MkPending* pending);");
+PL_CALL(inputs_attn, "inputs_attn", "extern \"C\" __device__ void pipelink_call_inputs_attn(const void* view, MkPending* pending);");
 PL_SERVE(op_attn, "op_attn");
 PL_CALL(rope_apply, "rope_apply", "extern \"C\" __device__ float pipelink_call_rope_apply(const void* view, const float* v, int i);");
 PL_USES("pipelink_mk_vec");

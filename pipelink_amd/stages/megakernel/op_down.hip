@@ -4,19 +4,23 @@
 #ifndef PIPELINK_EMIT
 #include "mk_device.hpp"
 
-extern "C" __device__ void mk_down_op(const void* view, const MkInstr* instr) {
+extern "C" __device__ void pipelink_call_inputs_down(const void* view, MkPending* pending);
+
+extern "C" __device__ void mk_down_op(const void* view, const MkInstr* instr, MkPending* pending) {
   const MkModel& m = mk::model(view);
   float* hv = mk::vec();
   float* scratch = hv + 8192;  // behind the vector
   const uint16_t* w = mk::layer_of(m, instr->layer).wdown;
   int first, last;
   mk::my_rows(m.d, first, last);
-  // the intermediate, this workgroup's first eight rows of the matrix and the residual they add to: all on their way at once
+  // this workgroup's first eight rows of the matrix are asked for first (they depend on nobody); then, once the other
+  // workgroups' intermediate is there, the intermediate and the residual the rows add to: all on their way at once
+  mk::v4i wreg[8][4];
+  if (first + 8 <= last) mk::split_load<8>(w + (int64_t)first * m.dff, m.dff, wreg);
+  pipelink_call_inputs_down(view, pending);
   mk::v4f hreg[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) hreg[j] = mk::shared_load4(m.h, 4 * (int)threadIdx.x + 4 * MK_THREADS * j, m.dff);  // past DFF: zeros
-  mk::v4i wreg[8][4];
-  if (first + 8 <= last) mk::split_load<8>(w + (int64_t)first * m.dff, m.dff, wreg);
   float xold = (int)threadIdx.x < 8 && first + (int)threadIdx.x < last ? mk::shared_load(m.x + first + threadIdx.x) : 0.0f;
 #pragma unroll
   for (int j = 0; j < 8; ++j)
@@ -40,7 +44,8 @@ PL_STAGE("mk.down", "0.1.0");
 PL_NO_PARAMS();
 PL_TOPOLOGY(true, "static");
 PL_VARIANT(0, {});
-PL_EXPORT(op_down, mk_down_op, "extern \"C\" __device__ void mk_down_op(const void* view, const MkInstr* instr);");
+PL_EXPORT(op_down, mk_down_op, "extern \"C\" __device__ void mk_down_op(const void* view, const MkInstr* instr, MkPending* pending);");
+PL_CALL(inputs_down, "inputs_down", "extern \"C\" __device__ void pipelink_call_inputs_down(const void* view, MkPending* pending);");
 PL_SERVE(op_down, "op_down");
 PL_USES("pipelink_mk_vec");
 // the number(s) the instruction stream calls this op by: one slot each in the link's opcode domain

@@ -3,14 +3,16 @@
 #ifndef PIPELINK_EMIT
 #include "mk_device.hpp"
 
-extern "C" __device__ void mk_lmhead_op(const void* view, const MkInstr* instr) {
+extern "C" __device__ void pipelink_call_inputs_lmhead(const void* view, MkPending* pending);
+
+extern "C" __device__ void mk_lmhead_op(const void* view, const MkInstr* instr, MkPending* pending) {
   (void)instr;
   const MkModel& m = mk::model(view);
   const uint16_t* w = mk::lm_head(m);
   const float* x = mk::vec();
   int first, last;
   mk::my_rows(m.vocab, first, last);
-  mk::matvec<4>(w, m.d, x, first, last, [&](int r, float v) { m.logits[r] = v; });
+  mk::matvec<4>(w, m.d, x, first, last, [&](int r, float v) { m.logits[r] = v; }, [&] { pipelink_call_inputs_lmhead(view, pending); });
 }
 #else
 #include "include/mk_abi.h"
@@ -20,7 +22,8 @@ PL_STAGE("mk.lmhead", "0.1.0");
 PL_NO_PARAMS();
 PL_TOPOLOGY(true, "static");
 PL_VARIANT(0, {});
-PL_EXPORT(op_lmhead, mk_lmhead_op, "extern \"C\" __device__ void mk_lmhead_op(const void* view, const MkInstr* instr);");
+PL_EXPORT(op_lmhead, mk_lmhead_op, "extern \"C\" __device__ void mk_lmhead_op(const void* view, const MkInstr* instr, MkPending* pending);");
+PL_CALL(inputs_lmhead, "inputs_lmhead", "extern \"C\" __device__ void pipelink_call_inputs_lmhead(const void* view, MkPending* pending);");
 PL_SERVE(op_lmhead, "op_lmhead");
 PL_USES("pipelink_mk_vec");
 // the number(s) the instruction stream calls this op by: one slot each in the link's opcode domain

@@ -5,7 +5,9 @@
 #ifndef PIPELINK_EMIT
 #include "mk_device.hpp"
 
-extern "C" __device__ void mk_oproj_op(const void* view, const MkInstr* instr) {
+extern "C" __device__ void pipelink_call_inputs_oproj(const void* view, MkPending* pending);
+
+extern "C" __device__ void mk_oproj_op(const void* view, const MkInstr* instr, MkPending* pending) {
   const MkModel& m = mk::model(view);
   float* a = mk::vec();
   const int n = m.hq * MK_HEAD_DIM, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -16,10 +18,16 @@ extern "C" __device__ void mk_oproj_op(const void* view, const MkInstr* instr) {
   const uint16_t* w = mk::layer_of(m, instr->layer).wo;
   int first, last;
   mk::my_rows(m.d, first, last);
-  // Everything this op reads from memory is asked for before anything is used: the chunks' maxima and sums, the
-  // first eight chunks of the partial outputs (two items of four floats per thread), the wave's first two matrix
-  // rows and the residual they add to.
+  // Everything this op reads from memory is asked for before anything is used: the wave's first two matrix rows
+  // (before the attention workgroups are waited for: the rows depend on nobody), then the chunks' maxima and sums,
+  // the first eight chunks of the partial outputs (two items of four floats per thread) and the residual the
+  // rows add to.
   constexpr int R = 2, CHUNKS_AHEAD = 8, ITEMS = 2;
+  const int row0 = first + R * wave;
+  mk::v4i wreg[R][4];
+  const bool rows_ahead = row0 + R <= last;
+  if (rows_ahead) mk::rows_load<R>(w + (int64_t)row0 * n, n, n, lane, wreg);
+  pipelink_call_inputs_oproj(view, pending);
   mk::v4f stat = {0.0f, 0.0f, 0.0f, 0.0f};
   if (tid < pairs) stat = mk::shared_load4(m.attn_partial, tid * MK_PARTIAL_STRIDE + MK_HEAD_DIM, count);
   mk::v4f part[ITEMS][CHUNKS_AHEAD];
@@ -30,12 +38,8 @@ extern "C" __device__ void mk_oproj_op(const void* view, const MkInstr* instr) {
     for (int c = 0; c < CHUNKS_AHEAD; ++c)  // an index past the buffer reads zeros
       part[it][c] = mk::shared_load4(m.attn_partial, item < n / 4 && c < m.chunks ? (head * m.chunks + c) * MK_PARTIAL_STRIDE + d : count, count);
   }
-  const int row0 = first + R * wave;
-  mk::v4i wreg[R][4];
   float xold[R] = {};
-  const bool rows_ahead = row0 + R <= last;
   if (rows_ahead) {
-    mk::rows_load<R>(w + (int64_t)row0 * n, n, n, lane, wreg);
 #pragma unroll
     for (int i = 0; i < R; ++i) xold[i] = mk::shared_load(m.x + row0 + i);
   }
@@ -100,7 +104,8 @@ PL_STAGE("mk.oproj", "0.1.0");
 PL_NO_PARAMS();
 PL_TOPOLOGY(true, "static");
 PL_VARIANT(0, {});
-PL_EXPORT(op_oproj, mk_oproj_op, "extern \"C\" __device__ void mk_oproj_op(const void* view, const MkInstr* instr);");
+PL_EXPORT(op_oproj, mk_oproj_op, "extern \"C\" __device__ void mk_oproj_op(const void* view, const MkInstr* instr, MkPending* pending);");
+PL_CALL(inputs_oproj, "inputs_oproj", "extern \"C\" __device__ void pipelink_call_inputs_oproj(const void* view, MkPending* pending);");
 PL_SERVE(op_oproj, "op_oproj");
 PL_USES("pipelink_mk_vec");
 // the number(s) the instruction stream calls this op by: one slot each in the link's opcode domain

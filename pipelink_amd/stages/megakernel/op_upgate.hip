@@ -3,7 +3,9 @@
 #ifndef PIPELINK_EMIT
 #include "mk_device.hpp"
 
-extern "C" __device__ void mk_upgate_op(const void* view, const MkInstr* instr) {
+extern "C" __device__ void pipelink_call_inputs_upgate(const void* view, MkPending* pending);
+
+extern "C" __device__ void mk_upgate_op(const void* view, const MkInstr* instr, MkPending* pending) {
   const MkModel& m = mk::model(view);
   const mk::Layer l = mk::layer_of(m, instr->layer);
   const float* x = mk::vec();
@@ -11,9 +13,15 @@ extern "C" __device__ void mk_upgate_op(const void* view, const MkInstr* instr) 
   int first, last;
   mk::my_rows(m.dff, first, last);
   constexpr int R = 4;
-  for (int r = first + R * wave; r < last; r += 4 * R) {  // DFF / workgroups is a multiple of 4 (the host checks)
+  // the wave's first four gate rows are asked for before the vector they multiply is waited for
+  mk::v4i ahead[R][4];
+  const int r0 = first + R * wave;
+  if (r0 < last) mk::rows_load<R>(l.wgate + (int64_t)r0 * m.d, m.d, m.d, lane, ahead);
+  pipelink_call_inputs_upgate(view, pending);
+  for (int r = r0; r < last; r += 4 * R) {  // DFF / workgroups is a multiple of 4 (the host checks)
     float g[R], u[R];
-    mk::rows_dot<R>(l.wgate + (int64_t)r * m.d, m.d, x, m.d, lane, g);
+    if (r == r0) mk::rows_dot<R>(l.wgate + (int64_t)r * m.d, m.d, x, m.d, lane, g, &ahead);
+    else mk::rows_dot<R>(l.wgate + (int64_t)r * m.d, m.d, x, m.d, lane, g);
     mk::rows_dot<R>(l.wup + (int64_t)r * m.d, m.d, x, m.d, lane, u);
     if (lane == 0) {
 #pragma unroll
@@ -30,7 +38,8 @@ PL_STAGE("mk.upgate", "0.1.0");
 PL_NO_PARAMS();
 PL_TOPOLOGY(true, "static");
 PL_VARIANT(0, {});
-PL_EXPORT(op_upgate, mk_upgate_op, "extern \"C\" __device__ void mk_upgate_op(const void* view, const MkInstr* instr);");
+PL_EXPORT(op_upgate, mk_upgate_op, "extern \"C\" __device__ void mk_upgate_op(const void* view, const MkInstr* instr, MkPending* pending);");
+PL_CALL(inputs_upgate, "inputs_upgate", "extern \"C\" __device__ void pipelink_call_inputs_upgate(const void* view, MkPending* pending);");
 PL_SERVE(op_upgate, "op_upgate");
 PL_USES("pipelink_mk_vec");
 // the number(s) the instruction stream calls this op by: one slot each in the link's opcode domain
