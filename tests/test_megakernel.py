@@ -123,13 +123,15 @@ def _bits(t: torch.Tensor) -> np.ndarray:
     return t.contiguous().view(torch.int16).numpy().view(np.uint16)
 
 
-def _run(paths_key, cfg, weights, cache, x, workgroups, image_key=None, time_launches=0):
+def _run(paths_key, cfg, weights, cache, x, workgroups, image_key=None, time_launches=0, program=None):
     from pipelink_amd.host.megakernel import open_session
 
     paths = mk_build.images()
     sess = open_session(paths[paths_key], _bits(weights), _bits(cache), x.numpy(), workgroups=workgroups, **cfg,
                         image=paths[image_key] if image_key else None)
     try:
+        if program is not None:
+            sess.write("program", program(sess.read("program")))
         sess.launch()
         sess.synchronize()
         out = {n: sess.read(n) for n in ("logits", "x", "kv_cache", "sync")}
@@ -165,6 +167,18 @@ def test_small_model_matches_the_oracle_linked_one_unit_and_swapped():
     assert all(np.array_equal(control[n], got[n]) for n in ("logits", "x", "kv_cache")), "linked and one-unit images differ"
     rebound = _run("rebind_link_json", cfg, weights, cache, x, workgroups=32)   # other opcode numbers, same packages
     assert all(np.array_equal(rebound[n], got[n]) for n in ("logits", "x", "kv_cache")), "rebound opcodes changed the result"
+    # The barrier's two halves and the held-back normalisation, off the beaten path: the step's last two instructions
+    # (final norm, LM head) replaced by an opcode nobody claimed with a barrier behind it (the interpreter itself has to
+    # wait for the barrier the down projection opened) and a normalisation as the very last instruction (held back, and
+    # nobody asks for it).  x and the cache must come out as from the whole step, the counters back at zero.
+    def detour(prog):
+        prog = prog.copy()
+        prog[-2] = (0, 0, 1, 0)
+        prog[-1] = prog[-5]                      # rmsnorm_ffn of the last layer (it writes only LDS)
+        return prog
+    off_path = _run("link_json", cfg, weights, cache, x, workgroups=32, program=detour)
+    assert list(off_path["sync"][:3]) == [0, 0, 0]
+    assert np.array_equal(off_path["x"], got["x"]) and np.array_equal(off_path["kv_cache"], got["kv_cache"])
     swapped = _run("swap_link_json", cfg, weights, cache, x, workgroups=32)
     assert list(swapped["sync"][:3]) == [0, 0, 0]
     assert _rel(swapped["logits"], got["logits"]) <= 1e-4 and _rel(swapped["logits"], want_logits.numpy()) <= 2e-3
