@@ -153,8 +153,22 @@ def _finalise(bitcode: Path, hsaco: Path, arch: str) -> None:
         _run([LLVM_BIN / "clang", "-x", "ir", "-target", "amdgcn-amd-amdhsa", f"-mcpu={arch}", "-O3", "-nogpulib",
               optimised, "-o", hsaco], "link.codegen")
         text = _run([LLVM_BIN / "llvm-objdump", "-d", "--no-show-raw-insn", hsaco], "audit.disassemble")
-        if not re.search(r"\bs_swappc_b64\b|\bs_setpc_b64\b", text):
+        if not seam_calls(text):
             break
+
+
+_LONG_BRANCH = re.compile(r"s_getpc_b64 (s\[\d+:\d+\])\s*\n\s*s_add_u32 s\d+, s\d+, (?:0x[0-9a-f]+|\d+)\s*\n\s*s_addc_u32 s\d+, s\d+, (?:0x[0-9a-f]+|-?\d+)\s*\n"
+                          r"\s*s_setpc_b64 \1")
+
+
+def seam_calls(disassembly: str) -> int:
+    """Calls and returns left in a disassembled image (``llvm-objdump -d --no-show-raw-insn``): ``s_swappc_b64``, and
+    ``s_setpc_b64`` unless it is the tail of a long branch -- past +-128 KB the compiler writes a branch as
+    ``s_getpc_b64; s_add_u32 <constant>; s_addc_u32; s_setpc_b64``, which leaves the function no more than a
+    ``s_branch`` does."""
+    text = re.sub(r"[ \t]*//[^\n]*", "", disassembly)
+    calls = len(re.findall(r"\bs_swappc_b64\b", text))
+    return calls + len(re.findall(r"\bs_setpc_b64\b", text)) - len(_LONG_BRANCH.findall(text))
 
 
 def audit(hsaco: Path) -> dict[str, int]:
@@ -165,7 +179,7 @@ def audit(hsaco: Path) -> dict[str, int]:
         m = re.search(rf"\.{key}:\s+(\d+)", notes)
         out[key] = int(m.group(1)) if m else 0
     text = _run([LLVM_BIN / "llvm-objdump", "-d", "--no-show-raw-insn", hsaco], "audit.disassemble")
-    out["calls"] = len(re.findall(r"\bs_swappc_b64\b|\bs_setpc_b64\b", text))
+    out["calls"] = seam_calls(text)
     out["mfma"] = len(re.findall(r"\bv_mfma_", text))
     out["instructions"] = sum(1 for line in text.splitlines() if re.match(r"\s+[sv]_|\s+ds_|\s+global_|\s+flat_|\s+buffer_|\s+scratch_", line))
     return out

@@ -15,6 +15,15 @@ extern "C" __device__ void mk_rmsnorm_op(const void* view, const MkInstr* instr)
   float* out = mk::vec();
   float* scratch = out + m.d;  // 4 floats behind the vector (the vector region holds at least D + 64 floats)
   const int tid = threadIdx.x;
+  // a thread normalises the elements it loads (four at a time), and asks for their weights in the same breath: one
+  // trip to memory, not two (the first 2048 elements' weights; longer vectors fetch the rest when they get there)
+  constexpr int AHEAD = 2;
+  uint2 wreg[AHEAD];
+#pragma unroll
+  for (int j = 0; j < AHEAD; ++j) {
+    const int i = 4 * tid + 4 * MK_THREADS * j;
+    wreg[j] = i < m.d ? *reinterpret_cast<const uint2*>(weight + i) : uint2{0u, 0u};
+  }
   float ss = 0.0f;
   for (int i = 4 * tid; i < m.d; i += 4 * MK_THREADS) {  // D is a multiple of 512
     const mk::v4f v = mk::shared_load4(m.x, i, m.d);
@@ -25,7 +34,21 @@ extern "C" __device__ void mk_rmsnorm_op(const void* view, const MkInstr* instr)
   if ((tid & 63) == 0) scratch[tid >> 6] = ss;
   __syncthreads();
   const float inv = __builtin_amdgcn_rsqf((scratch[0] + scratch[1] + scratch[2] + scratch[3]) / (float)m.d + m.eps);
-  for (int i = tid; i < m.d; i += MK_THREADS) out[i] = out[i] * inv * mk::bf16_to_f32(weight[i]);
+#pragma unroll
+  for (int j = 0; j < AHEAD; ++j) {
+    const int i = 4 * tid + 4 * MK_THREADS * j;
+    if (i < m.d) {
+      const mk::v4f v = *reinterpret_cast<const mk::v4f*>(out + i);  // this thread's own four
+      *reinterpret_cast<mk::v4f*>(out + i) = mk::v4f{v.x * inv * mk::bf16_to_f32(wreg[j].x & 0xFFFFu), v.y * inv * __uint_as_float(wreg[j].x & 0xFFFF0000u),
+                                                     v.z * inv * mk::bf16_to_f32(wreg[j].y & 0xFFFFu), v.w * inv * __uint_as_float(wreg[j].y & 0xFFFF0000u)};
+    }
+  }
+  for (int i = 4 * tid + 4 * MK_THREADS * AHEAD; i < m.d; i += 4 * MK_THREADS) {
+    const mk::v4f v = *reinterpret_cast<const mk::v4f*>(out + i);
+    const uint2 w = *reinterpret_cast<const uint2*>(weight + i);
+    *reinterpret_cast<mk::v4f*>(out + i) = mk::v4f{v.x * inv * mk::bf16_to_f32(w.x & 0xFFFFu), v.y * inv * __uint_as_float(w.x & 0xFFFF0000u),
+                                                   v.z * inv * mk::bf16_to_f32(w.y & 0xFFFFu), v.w * inv * __uint_as_float(w.y & 0xFFFF0000u)};
+  }
 }
 #else
 #include "include/mk_abi.h"

@@ -106,3 +106,19 @@ def test_linked_image_passes_the_gate_against_the_one_unit_control(pair):
     assert max(r["private_segment_fixed_size"] for r in report["resources"].values()) <= isagate.SPILL_LIMIT_BYTES
     text = isagate.summary(report)
     assert "gate passed: True" in text and "v_mfma" in text
+
+
+def test_link_audit_tells_a_long_branch_from_a_call():
+    """An image larger than a branch's reach (+-128 KB) jumps with s_getpc / s_add / s_addc / s_setpc: not a seam call."""
+    from pipelink_amd.pipec.linker import seam_calls
+
+    long_branch = ("\ts_cbranch_scc0 6   // 00194C: BF840006 <pipelink_kernel+0x68>\n"
+                   "\ts_getpc_b64 s[98:99]                                       // 000000001950: BEE21C00\n"
+                   "\ts_add_u32 s98, s98, 0x1ff0c                                // 000000001954: 8062FF62 0001FF0C\n"
+                   "\ts_addc_u32 s99, s99, 0                                     // 00000000195C: 8263FF63 00000000\n"
+                   "\ts_setpc_b64 s[98:99]                                       // 000000001964: BE801D62\n")
+    assert seam_calls(long_branch) == 0
+    call = ("\ts_getpc_b64 s[4:5]\n\ts_add_u32 s4, s4, 0x10\n\ts_addc_u32 s5, s5, 0\n\ts_swappc_b64 s[30:31], s[4:5]\n")
+    assert seam_calls(call) == 1
+    assert seam_calls("\tv_add_f32 v0, v0, v1\n\ts_setpc_b64 s[30:31]\n") == 1                      # a return: somebody was called
+    assert seam_calls(long_branch.replace("s_setpc_b64 s[98:99]", "s_setpc_b64 s[30:31]")) == 1  # not the pc it just computed
