@@ -107,7 +107,8 @@ __device__ __forceinline__ void rows_load(const uint16_t* rows, int64_t pitch, i
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const v4i zero = {0, 0, 0, 0};
-      w[r][j] = c0 + 64 * j < n / 8 ? *reinterpret_cast<const v4i*>(rows + r * pitch + 8 * (c0 + 64 * j)) : zero;
+      // weights pass through once per token: loaded as non-temporal, they do not push the activations out of the L2
+      w[r][j] = c0 + 64 * j < n / 8 ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(rows + r * pitch + 8 * (c0 + 64 * j))) : zero;
     }
 }
 template <int R>
