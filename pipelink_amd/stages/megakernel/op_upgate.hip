@@ -13,16 +13,20 @@ extern "C" __device__ void mk_upgate_op(const void* view, const MkInstr* instr, 
   int first, last;
   mk::my_rows(m.dff, first, last);
   constexpr int R = 4;
-  // the wave's first four gate rows are asked for before the vector they multiply is waited for
-  mk::v4i ahead[R][4];
+  // Two sets of row registers, gate and up, each refilled with the wave's next four rows as soon as it has been used:
+  // one set is always on its way.  The first gate rows are asked for before the vector they multiply is waited for.
+  mk::v4i wg[R][4], wu[R][4];
   const int r0 = first + R * wave;
-  if (r0 < last) mk::rows_load<R>(l.wgate + (int64_t)r0 * m.d, m.d, m.d, lane, ahead);
+  if (r0 < last) mk::rows_load<R>(l.wgate + (int64_t)r0 * m.d, m.d, m.d, lane, wg);
   pipelink_call_inputs_upgate(view, pending);
+  if (r0 < last) mk::rows_load<R>(l.wup + (int64_t)r0 * m.d, m.d, m.d, lane, wu);
   for (int r = r0; r < last; r += 4 * R) {  // DFF / workgroups is a multiple of 4 (the host checks)
+    const int next = r + 4 * R;
     float g[R], u[R];
-    if (r == r0) mk::rows_dot<R>(l.wgate + (int64_t)r * m.d, m.d, x, m.d, lane, g, &ahead);
-    else mk::rows_dot<R>(l.wgate + (int64_t)r * m.d, m.d, x, m.d, lane, g);
-    mk::rows_dot<R>(l.wup + (int64_t)r * m.d, m.d, x, m.d, lane, u);
+    mk::rows_dot<R>(l.wgate + (int64_t)r * m.d, m.d, x, m.d, lane, g, &wg);
+    if (next < last) mk::rows_load<R>(l.wgate + (int64_t)next * m.d, m.d, m.d, lane, wg);
+    mk::rows_dot<R>(l.wup + (int64_t)r * m.d, m.d, x, m.d, lane, u, &wu);
+    if (next < last) mk::rows_load<R>(l.wup + (int64_t)next * m.d, m.d, m.d, lane, wu);
     if (lane == 0) {
 #pragma unroll
       for (int i = 0; i < R; ++i)
