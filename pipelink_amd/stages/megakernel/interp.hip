@@ -56,7 +56,12 @@ __device__ __forceinline__ bool poll(uint32_t* word, uint32_t target, bool local
       const uint32_t zero = 0;
       asm volatile("global_atomic_add %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)" : "=&v"(seen) : "v"(word), "v"(zero) : "memory");
     } else {
+      // two loads in flight, a fraction of a round trip apart: the answer is half a round trip old on average, not a whole one
       seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_s_sleep(4);
+      const uint32_t later = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if ((int32_t)(seen - target) >= 0) return true;
+      seen = later;
     }
     if ((int32_t)(seen - target) >= 0) return true;
     __builtin_amdgcn_s_sleep(1);
