@@ -150,6 +150,30 @@ def test_window_mask_matches_the_oracle_on_every_head(window):
 
 
 @pytest.mark.gpu
+def test_window_mask_at_the_stated_size_on_sampled_heads():
+    """B 4, 32 / 8 heads, S 4096 with a window of 1024 keys: tiles start streaming at their first visible block."""
+    from pipelink_amd.host.attention import open_session
+
+    B, HQ, HKV, S, W = 4, 32, 8, 4096, 1024
+    q, k, v = oa.inputs(B, HQ, HKV, S, seed=0)
+    sess = open_session(fa_build.images()["window_link_json"], _bits(q), _bits(k), _bits(v), window=W)
+    try:
+        sess.write("o", np.full((B, S, HQ * 128), 0x7FC0, dtype=np.uint16))
+        sess.launch()
+        sess.synchronize()
+        o = _from_bits(sess.read("o"))
+        ms = sorted(sess.time(50) for _ in range(3))[1]
+        print(f"attention, window {W}: {ms:.3f} ms", flush=True)
+    finally:
+        sess.close()
+    for (b, h), want in oa.attention(q, k, v, [(0, 5), (2, 17)], window=W).items():
+        got = o[b, :, h * 128:(h + 1) * 128]
+        assert torch.isfinite(got).all()
+        assert (got - want).abs().max().item() <= 1e-2 * want.abs().max().item(), (b, h)
+        assert ((got - want).norm() / want.norm()).item() <= 1e-2, (b, h)
+
+
+@pytest.mark.gpu
 def test_stated_case_sampled_heads_one_unit_control_and_output_projection():
     from pipelink_amd.host.attention import open_session
     from pipelink_amd.host.one_epilogue import open_session as open_gemm
