@@ -73,6 +73,18 @@ int plk_mok_session_destroy(plk_mok_session* s);
 int plk_mok_forward(plk_mok_session* s, const plk_mok_problem* p, void* stream);
 int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass, void* stream);
 
+/* plk_mok_forward for callers that cannot allocate or wait: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  It calls no hipMalloc / hipFree and no
+ * allocating library routine, copies nothing from host memory and never synchronises: the params images the kernels
+ * read (at most PLK_MOK_STATIC_IMAGE_BYTES per pass, else PLK_E_CAPACITY) are stored by a small kernel, ahead of the
+ * two passes in stream order, into a fixed area of device memory that belongs to the library (2 x
+ * PLK_MOK_STATIC_IMAGE_BYTES per GPU, held until the process ends; its address is resolved when a session is
+ * created on that GPU).  The session's device must be the current one.  Every call on a GPU shares that GPU's
+ * area: calls that overlap on one GPU (two streams, two threads) race on it; calls in one stream do not.
+ * Results are byte for byte those of plk_mok_forward. */
+#define PLK_MOK_STATIC_IMAGE_BYTES 1024
+int plk_mok_forward_static(plk_mok_session* s, const plk_mok_problem* p, void* stream);
+
 /* MXFP8 block quantiser on the device (what ops.mxfp8_quantize does for the reference's
  * harness, campaigns/mok/host/mok_port_host.py:122): src is fp32 (src_is_bf16 = 0) or bf16
  * [rows, k], dst_q [rows, ld_q] e4m3 (ld_q >= k; pad bytes untouched), dst_sc [rows, ld_sc] e8m0

@@ -8,6 +8,7 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -24,6 +25,7 @@ struct plk_mok_session {
   uint64_t params_dev[2] = {0, 0};            // device copies of the two passes' params images
   std::vector<unsigned char> params_host[2];  // what the device copies hold
   int32_t compute_units = 0;
+  int device = 0;  // the device that was current when the session was created
 };
 
 static plk_mok::Dims dims_of(const plk_mok_problem* p, int pass) {
@@ -59,6 +61,66 @@ static int check_problem(const plk_mok_problem* p) {
   return PLK_OK;
 }
 
+
+// One pass's params image: the three owners' records at their linked offsets, zeros between them.
+static void fill_image(const plk_mok_link_info& link, const plk_mok_problem* p, int pass, unsigned char* image) {
+  const plk_mok::Dims d = dims_of(p, pass);
+  const MokFrameworkParams fw = plk_mok::framework_params(d, p->tokens_per_expert);
+  const MokGemmResidue g = plk_mok::gemm_residue(
+      d, plk_mok::GemmAddresses{p->x_q, p->x_sc, p->w_gate_q, p->w_gate_sc, p->w_up_q, p->w_up_sc, p->w_down_q, p->w_down_sc,
+                                p->hidden_q, p->hidden_sc, p->y, p->row_token});
+  const MokActResidue a = plk_mok::act_residue(d, p->hidden_q, p->hidden_sc);
+  std::memcpy(image + link.framework_offset, &fw, sizeof fw);
+  std::memcpy(image + link.gemm_offset, &g, sizeof g);
+  std::memcpy(image + link.act_offset, &a, sizeof a);
+}
+
+// Launch of one pass on a params image that is already on the device.  Persistent grid: the solved occupancy
+// on every CU, a multiple of the XCD count, but no more workgroups than there can be tiles.
+static int launch_pass(plk_mok_session* s, const plk_mok_problem* p, int pass, void* stream, uint64_t params_dev) {
+  const plk_mok::Dims d = dims_of(p, pass);
+  const int64_t max_tiles = plk_mok::max_workgroups(d);
+  int64_t wgs = (int64_t)s->compute_units * s->link.workgroups_per_cu;
+  if (wgs > max_tiles) wgs = max_tiles;
+  wgs = (wgs + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
+  const uint32_t grid[3] = {(uint32_t)wgs, 1, 1};
+  const uint32_t block[3] = {s->link.threads, 1, 1};
+  return plk_hip_launch(s->kernel, grid, block, s->link.dyn_lds_bytes, stream, params_dev);
+}
+
+// ---- device memory of the entry point that allocates nothing (plk_mok_forward_static) -------------------
+// The two passes' params images, PLK_MOK_STATIC_IMAGE_BYTES each, live in this file-scope array: every GPU
+// the library runs on holds its own copy, at its own address, until the process ends.  `scratch` is only a
+// name on the host; the address kernels are given is what hipGetSymbolAddress returned for the device that
+// was current, kept per device in g_static_area.
+constexpr int STATIC_WORDS = 2 * PLK_MOK_STATIC_IMAGE_BYTES / 4;
+static __device__ __align__(256) unsigned char scratch[2 * PLK_MOK_STATIC_IMAGE_BYTES];
+constexpr int MAX_DEVICES = 64;
+static unsigned char* g_static_area[MAX_DEVICES];
+static std::mutex g_static_mutex;
+
+struct StaticImages {
+  uint32_t words[STATIC_WORDS];
+};
+__global__ void __launch_bounds__(STATIC_WORDS) plk_mok_store_images(StaticImages images, uint32_t* dst) {
+  dst[threadIdx.x] = images.words[threadIdx.x];
+}
+
+// once per device, with that device current
+static int resolve_static_area(int dev) {
+  if (dev < 0 || dev >= MAX_DEVICES) return plk_hip_set_error(PLK_E_CAPACITY, "plk_mok: device ordinal beyond 63");
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (g_static_area[dev]) return PLK_OK;
+  void* ptr = nullptr;
+  const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !ptr) {
+    (void)hipGetLastError();
+    return plk_hip_set_error(PLK_E_RESOURCE, "plk_mok: hipGetSymbolAddress of the static params area failed");
+  }
+  g_static_area[dev] = static_cast<unsigned char*>(ptr);
+  return PLK_OK;
+}
+
 extern "C" {
 
 int plk_mok_session_create(const void* image, size_t image_bytes, const plk_mok_link_info* link,
@@ -87,6 +149,8 @@ int plk_mok_session_create(const void* image, size_t image_bytes, const plk_mok_
     plk_hip_device_info info;
     rc = plk_hip_device_info_get(dev, &info);
     s->compute_units = info.compute_units;
+    s->device = dev;
+    if (rc == PLK_OK) rc = resolve_static_area(dev);
   }
   if (rc != PLK_OK) {
     plk_mok_session_destroy(s);
@@ -113,18 +177,9 @@ int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass,
   if (rc != PLK_OK) return rc;
   if (p->routed_rows == 0) return PLK_OK;  // nothing routed to this rank
 
-  const plk_mok::Dims d = dims_of(p, pass);
-  const MokFrameworkParams fw = plk_mok::framework_params(d, p->tokens_per_expert);
-  const MokGemmResidue g = plk_mok::gemm_residue(
-      d, plk_mok::GemmAddresses{p->x_q, p->x_sc, p->w_gate_q, p->w_gate_sc, p->w_up_q, p->w_up_sc, p->w_down_q, p->w_down_sc,
-                                p->hidden_q, p->hidden_sc, p->y, p->row_token});
-  const MokActResidue a = plk_mok::act_residue(d, p->hidden_q, p->hidden_sc);
-
   const int slot = pass - 1;
   std::vector<unsigned char> image(s->link.params_bytes, 0);
-  std::memcpy(image.data() + s->link.framework_offset, &fw, sizeof fw);
-  std::memcpy(image.data() + s->link.gemm_offset, &g, sizeof g);
-  std::memcpy(image.data() + s->link.act_offset, &a, sizeof a);
+  fill_image(s->link, p, pass, image.data());
   if (image != s->params_host[slot]) {
     // a new problem: its params image goes to the device first, which synchronises and cannot be part of a graph
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
@@ -135,21 +190,40 @@ int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass,
     if (rc != PLK_OK) return rc;
     s->params_host[slot].swap(image);
   }
-
-  // persistent grid: the solved occupancy on every CU, a multiple of the XCD count, but no
-  // more workgroups than there can be tiles
-  const int64_t max_tiles = plk_mok::max_workgroups(d);
-  int64_t wgs = (int64_t)s->compute_units * s->link.workgroups_per_cu;
-  if (wgs > max_tiles) wgs = max_tiles;
-  wgs = (wgs + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
-  const uint32_t grid[3] = {(uint32_t)wgs, 1, 1};
-  const uint32_t block[3] = {s->link.threads, 1, 1};
-  return plk_hip_launch(s->kernel, grid, block, s->link.dyn_lds_bytes, stream, s->params_dev[slot]);
+  return launch_pass(s, p, pass, stream, s->params_dev[slot]);
 }
 
 int plk_mok_forward(plk_mok_session* s, const plk_mok_problem* p, void* stream) {
   int rc = plk_mok_forward_pass(s, p, 1, stream);
   if (rc == PLK_OK) rc = plk_mok_forward_pass(s, p, 2, stream);
+  return rc;
+}
+
+int plk_mok_forward_static(plk_mok_session* s, const plk_mok_problem* p, void* stream) {
+  if (!s) return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok_forward_static: null session");
+  int rc = check_problem(p);
+  if (rc != PLK_OK) return rc;
+  if (s->link.params_bytes > PLK_MOK_STATIC_IMAGE_BYTES)
+    return plk_hip_set_error(PLK_E_CAPACITY, "plk_mok_forward_static: the linked image's params exceed "
+                                             "PLK_MOK_STATIC_IMAGE_BYTES (1024) per pass");
+  if (p->routed_rows == 0) return PLK_OK;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev != s->device)
+    return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok_forward_static: the session's device must be the current one");
+  unsigned char* const base = g_static_area[dev];  // resolved when the session was created on this device
+  if (!base) return plk_hip_set_error(PLK_E_RESOURCE, "plk_mok_forward_static: the device's static area was not resolved");
+
+  // Both passes' params images travel as the argument of a small kernel that stores them into the static area:
+  // no copy from host memory, no wait, and stream order puts it in front of the two launches that read it.
+  StaticImages images;
+  std::memset(&images, 0, sizeof images);
+  for (int pass = 1; pass <= 2; ++pass)
+    fill_image(s->link, p, pass, reinterpret_cast<unsigned char*>(images.words) + (pass - 1) * PLK_MOK_STATIC_IMAGE_BYTES);
+  plk_mok_store_images<<<dim3(1), dim3(STATIC_WORDS), 0, (hipStream_t)stream>>>(images, reinterpret_cast<uint32_t*>(base));
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return plk_hip_set_error(PLK_E_RESOURCE, hipGetErrorString(e));
+  for (int pass = 1; pass <= 2 && rc == PLK_OK; ++pass)
+    rc = launch_pass(s, p, pass, stream, (uint64_t)(uintptr_t)(base + (pass - 1) * PLK_MOK_STATIC_IMAGE_BYTES));
   return rc;
 }
 

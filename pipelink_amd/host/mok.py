@@ -130,6 +130,12 @@ class MoKSession:
                           w_up_sc=w_up_sc.data_ptr(), w_down_q=w_down_q.data_ptr(), w_down_sc=w_down_sc.data_ptr(),
                           hidden_q=hidden_q.data_ptr(), hidden_sc=hidden_sc.data_ptr(), y=y.data_ptr())
 
+    def forward_static(self, problem: MokProblem, stream: int | None = None) -> None:
+        """Both passes through the entry point that allocates nothing (``plk_mok_forward_static``): the params images
+        go into a fixed area of device memory the library owns; calls that overlap on one GPU race on it."""
+        s = c_void_p(torch.cuda.current_stream().cuda_stream if stream is None else stream)
+        check(self.lib, self.lib.plk_mok_forward_static(self._handle, byref(problem), s))
+
     def forward(self, problem: MokProblem, stream: int | None = None, which: int = 0) -> None:
         """Launch both passes (``which=0``) or one of them (1 = gate/up+SwiGLU+requant, 2 = down)."""
         s = c_void_p(torch.cuda.current_stream().cuda_stream if stream is None else stream)
