@@ -208,13 +208,14 @@ typedef struct plk_session_v2 plk_session; /* provider-owned, opaque */
 #define MOK_SCALAR_INTERMEDIATE 3u       /* I = d_ff */
 #define MOK_SCALAR_NUM_LOCAL_EXPERTS 4u  /* E */
 #define MOK_SCALAR_SWIGLU_LIMIT 10u      /* f64 */
-#define MOK_SCALAR_PASS 11u              /* 1 = gate/up + SwiGLU + requant, 2 = down */
+#define MOK_SCALAR_PASS 11u              /* 0 = both GEMMs in one launch, 1 = gate/up + SwiGLU + requant, 2 = down */
 #define MOK_SCALAR_PRECISION 12u         /* 1 = MXFP8 (the only one built) */
 #define MOK_SCALAR_ROUTED_ROWS 60u       /* R = sum(tokens_per_expert) */
 #define MOK_SCALAR_LD_Q_H 61u            /* code row pitch of x, bytes */
 #define MOK_SCALAR_LD_Q_I 62u            /* code row pitch of hidden, bytes */
 #define MOK_SCALAR_LD_SC_H 63u           /* scale row pitch of x */
 #define MOK_SCALAR_LD_SC_I 64u           /* scale row pitch of hidden */
+#define MOK_SCALAR_WORKSPACE_WORDS 65u   /* 32 + ceil(R / 256) + E: words of the launch workspace */
 
 /* Channels of owner mok.gemm (channel_id = index + 1), all u8 unless noted:
  *   1 x_q [T, ld_q_h] R          2 x_sc [T, ld_sc_h] R
@@ -224,10 +225,13 @@ typedef struct plk_session_v2 plk_session; /* provider-owned, opaque */
  *   9 hidden_q [R, ld_q_i] R       10 hidden_sc [R, ld_sc_i] R
  *  11 y [R, H] bf16 W              12 row_token [R] i32 R (a zero-size resource = rows are tokens)
  * Channels of owner mok.act:       1 hidden_q [R, ld_q_i] W   2 hidden_sc [R, ld_sc_i] W
- * Channels of owner mok.framework: 1 tokens_per_expert [E] i32 R */
+ * Channels of owner mok.framework: 1 tokens_per_expert [E] i32 R
+ *                                  2 workspace [workspace_words] u32 W: status word and readiness counters of a launch;
+ *                                    all zero before the first launch, every launch leaves it zero again (but for
+ *                                    word 0, the sticky status: bit 0 = a bounded dependency wait gave up) */
 #define MOK_GEMM_CHANNEL_COUNT 12u
 #define MOK_ACT_CHANNEL_COUNT 2u
-#define MOK_FRAMEWORK_CHANNEL_COUNT 1u
+#define MOK_FRAMEWORK_CHANNEL_COUNT 2u
 
 /* Entry points, one set per owner suffix (reference: host ABI header :293-300 and
  * campaigns/mok/port/gemm/provider.cu:217-303).  `args` must be null: everything an owner

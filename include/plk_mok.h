@@ -66,23 +66,36 @@ typedef struct plk_mok_session plk_mok_session;
 
 int plk_mok_session_create(const void* image, size_t image_bytes, const plk_mok_link_info* link, plk_mok_session** out);
 int plk_mok_session_destroy(plk_mok_session* s);
-/* both passes; or one of them (pass 1 = gate/up + SwiGLU + requant, pass 2 = down).  The session keeps the params image
- * of the last problem per pass on the device: a call with the same problem only launches (and can be captured into a
- * graph); a call with another problem first uploads its image, which synchronises the stream -- on a stream that is
- * being captured that call returns PLK_E_CONTRACT. */
+/* The forward.  plk_mok_forward runs both GEMMs in ONE launch when every row of hidden_q is a whole number of
+ * 128-byte cache lines (hidden_q and ld_q_i multiples of 128): down tiles wait on per-row-tile readiness counters that
+ * the gate/up tiles bump (campaigns/mok/port/framework/interp_fwd.cu:174-213, gemm/gemm.cu:364-382 in the reference).
+ * With any other pitch it is two launches, pass 1 then pass 2.  plk_mok_forward_pass runs one of them (pass 1 = gate/up
+ * + SwiGLU + requant, pass 2 = down).  The session keeps the params image of the last problem per kind of launch on
+ * the device: a call with the same problem only launches (and can be captured into a graph); a call with another
+ * problem first uploads its image, which synchronises the stream -- on a stream that is being captured that call
+ * returns PLK_E_CONTRACT.  A problem with more routed-row tiles than any before also makes the session replace its
+ * launch workspace (device synchronisation, same rule under capture). */
 int plk_mok_forward(plk_mok_session* s, const plk_mok_problem* p, void* stream);
 int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass, void* stream);
 
+/* Waits for the stream, then returns and clears the sticky status of the session's launches: 0, or MOK_STATUS_* bits
+ * (bit 0: a down tile gave up waiting for its rows of `hidden` after 2^18 polls and multiplied what was there --
+ * the outputs of that forward are not to be trusted).  The waits are bounded so that a launch always ends. */
+int plk_mok_status(plk_mok_session* s, void* stream, uint32_t* status);
+
 /* plk_mok_forward for callers that cannot allocate or wait: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  No counterpart in the reference.  It calls no hipMalloc / hipFree and no
- * allocating library routine, copies nothing from host memory and never synchronises: the params images the kernels
- * read (at most PLK_MOK_STATIC_IMAGE_BYTES per pass, else PLK_E_CAPACITY) are stored by a small kernel, ahead of the
- * two passes in stream order, into a fixed area of device memory that belongs to the library (2 x
- * PLK_MOK_STATIC_IMAGE_BYTES per GPU, held until the process ends; its address is resolved when a session is
- * created on that GPU).  The session's device must be the current one.  Every call on a GPU shares that GPU's
- * area: calls that overlap on one GPU (two streams, two threads) race on it; calls in one stream do not.
+ * allocating library routine, copies nothing from host memory and never synchronises: what plk_mok_forward keeps in
+ * session-owned device buffers -- the launches' params images (at most PLK_MOK_STATIC_IMAGE_BYTES each, else
+ * PLK_E_CAPACITY) and the launch workspace of readiness counters (32 + ceil(routed_rows / 256) +
+ * num_experts words, at most PLK_MOK_STATIC_WORKSPACE_WORDS, else PLK_E_CAPACITY) -- lives in a fixed area of device
+ * memory that belongs to the library (66 KB per GPU, held until the process ends; its address is resolved when a
+ * session is created on that GPU) and is written by a small kernel ahead of the launches in stream order, which also
+ * clears the workspace.  The session's device must be the current one.  Every call on a GPU shares that GPU's area:
+ * calls that overlap on one GPU (two streams, two threads) race on it; calls in one stream do not.
  * Results are byte for byte those of plk_mok_forward. */
 #define PLK_MOK_STATIC_IMAGE_BYTES 1024
+#define PLK_MOK_STATIC_WORKSPACE_WORDS 16384
 int plk_mok_forward_static(plk_mok_session* s, const plk_mok_problem* p, void* stream);
 
 /* MXFP8 block quantiser on the device (what ops.mxfp8_quantize does for the reference's

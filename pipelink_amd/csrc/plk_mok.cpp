@@ -18,15 +18,23 @@ extern "C" int plk_hip_set_error(int code, const char* what);
 
 using plk_mok::NUM_XCD;
 
+constexpr int IMAGES = 3;  // params images a session keeps: both GEMMs in one launch (pass 0), pass 1, pass 2
+
 struct plk_mok_session {
   plk_hip_module* module = nullptr;
   plk_hip_function* kernel = nullptr;
   plk_mok_link_info link{};
-  uint64_t params_dev[2] = {0, 0};            // device copies of the two passes' params images
-  std::vector<unsigned char> params_host[2];  // what the device copies hold
+  uint64_t params_dev[IMAGES] = {0, 0, 0};         // device copies of the params images, by pass
+  std::vector<unsigned char> params_host[IMAGES];  // what the device copies hold
+  uint64_t workspace = 0;                          // readiness counters of a launch (device, zero between launches)
+  int64_t workspace_words = 0;
   int32_t compute_units = 0;
   int device = 0;  // the device that was current when the session was created
+  bool used_static = false;  // plk_mok_forward_static has run: the static area's status word counts too
 };
+
+// words the session's first workspace is made for (a problem that needs more gets a larger one)
+constexpr int64_t WORKSPACE_WORDS_AT_CREATE = 4096;
 
 static plk_mok::Dims dims_of(const plk_mok_problem* p, int pass) {
   plk_mok::Dims d;
@@ -62,10 +70,30 @@ static int check_problem(const plk_mok_problem* p) {
 }
 
 
+static bool stream_is_capturing(void* stream) {
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  return stream && hipStreamIsCapturing((hipStream_t)stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusActive;
+}
+
+// (re)places the session's workspace by one of at least `words` zeroed words
+static int make_workspace(plk_mok_session* s, int64_t words) {
+  if (s->workspace) {
+    int rc = plk_hip_free(s->workspace);
+    s->workspace = 0;
+    s->workspace_words = 0;
+    if (rc != PLK_OK) return rc;
+  }
+  int rc = plk_hip_alloc((size_t)words * 4, &s->workspace);
+  if (rc == PLK_OK) rc = plk_hip_zero(s->workspace, (size_t)words * 4, nullptr);
+  if (rc == PLK_OK) rc = plk_hip_synchronize(nullptr);
+  if (rc == PLK_OK) s->workspace_words = words;
+  return rc;
+}
+
 // One pass's params image: the three owners' records at their linked offsets, zeros between them.
-static void fill_image(const plk_mok_link_info& link, const plk_mok_problem* p, int pass, unsigned char* image) {
+static void fill_image(const plk_mok_link_info& link, const plk_mok_problem* p, int pass, uint64_t workspace, unsigned char* image) {
   const plk_mok::Dims d = dims_of(p, pass);
-  const MokFrameworkParams fw = plk_mok::framework_params(d, p->tokens_per_expert);
+  const MokFrameworkParams fw = plk_mok::framework_params(d, p->tokens_per_expert, workspace);
   const MokGemmResidue g = plk_mok::gemm_residue(
       d, plk_mok::GemmAddresses{p->x_q, p->x_sc, p->w_gate_q, p->w_gate_sc, p->w_up_q, p->w_up_sc, p->w_down_q, p->w_down_sc,
                                 p->hidden_q, p->hidden_sc, p->y, p->row_token});
@@ -89,21 +117,28 @@ static int launch_pass(plk_mok_session* s, const plk_mok_problem* p, int pass, v
 }
 
 // ---- device memory of the entry point that allocates nothing (plk_mok_forward_static) -------------------
-// The two passes' params images, PLK_MOK_STATIC_IMAGE_BYTES each, live in this file-scope array: every GPU
-// the library runs on holds its own copy, at its own address, until the process ends.  `scratch` is only a
-// name on the host; the address kernels are given is what hipGetSymbolAddress returned for the device that
-// was current, kept per device in g_static_area.
-constexpr int STATIC_WORDS = 2 * PLK_MOK_STATIC_IMAGE_BYTES / 4;
-static __device__ __align__(256) unsigned char scratch[2 * PLK_MOK_STATIC_IMAGE_BYTES];
+// What plk_mok_forward keeps in buffers the session allocates -- the params images of the launches (two at most,
+// PLK_MOK_STATIC_IMAGE_BYTES each) and the launch workspace (status word and readiness counters, up to
+// PLK_MOK_STATIC_WORKSPACE_WORDS words) -- lives in this file-scope array: every GPU the library runs on holds its
+// own copy, at its own address, until the process ends.  `scratch` is only a name on the host; the address
+// kernels are given is what hipGetSymbolAddress returned for the device that was current, kept per device in
+// g_static_area.
+constexpr int STATIC_IMAGE_WORDS = 2 * PLK_MOK_STATIC_IMAGE_BYTES / 4;
+constexpr size_t STATIC_WORKSPACE_OFFSET = 2 * PLK_MOK_STATIC_IMAGE_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_WORKSPACE_OFFSET + 4 * PLK_MOK_STATIC_WORKSPACE_WORDS];
 constexpr int MAX_DEVICES = 64;
 static unsigned char* g_static_area[MAX_DEVICES];
 static std::mutex g_static_mutex;
 
 struct StaticImages {
-  uint32_t words[STATIC_WORDS];
+  uint32_t words[STATIC_IMAGE_WORDS];
 };
-__global__ void __launch_bounds__(STATIC_WORDS) plk_mok_store_images(StaticImages images, uint32_t* dst) {
+// Stores the params images and puts the workspace words a launch of this size uses back to zero (a launch leaves them
+// zero, but one that was cut short would not have); word 0, the sticky status, is left alone.
+__global__ void __launch_bounds__(STATIC_IMAGE_WORDS) plk_mok_store_images(StaticImages images, uint32_t* dst, uint32_t* workspace,
+                                                                           int workspace_words) {
   dst[threadIdx.x] = images.words[threadIdx.x];
+  for (int w = 1 + threadIdx.x; w < workspace_words; w += STATIC_IMAGE_WORDS) workspace[w] = 0u;
 }
 
 // once per device, with that device current
@@ -139,10 +174,11 @@ int plk_mok_session_create(const void* image, size_t image_bytes, const plk_mok_
   s->link = *link;
   int rc = plk_hip_module_load(image, image_bytes, &s->module);
   if (rc == PLK_OK) rc = plk_hip_module_function(s->module, "pipelink_kernel", link->dyn_lds_bytes, &s->kernel);
-  for (int i = 0; i < 2 && rc == PLK_OK; ++i) {
+  for (int i = 0; i < IMAGES && rc == PLK_OK; ++i) {
     rc = plk_hip_alloc(link->params_bytes, &s->params_dev[i]);
     s->params_host[i].assign(link->params_bytes, 0xA5);  // differs from any real image: first call uploads
   }
+  if (rc == PLK_OK) rc = make_workspace(s, WORKSPACE_WORDS_AT_CREATE);
   if (rc == PLK_OK) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) dev = 0;
@@ -165,9 +201,37 @@ int plk_mok_session_destroy(plk_mok_session* s) {
   int rc = PLK_OK;
   for (uint64_t a : s->params_dev)
     if (a) { int r = plk_hip_free(a); if (r) rc = r; }
+  if (s->workspace) { int r = plk_hip_free(s->workspace); if (r) rc = r; }
   if (s->module) { int r = plk_hip_module_unload(s->module); if (r) rc = r; }
   delete s;
   return rc;
+}
+
+// One launch of the session's image: pass 0 = both GEMMs, 1 = gate/up + SwiGLU + requant, 2 = down.
+static int forward_launch(plk_mok_session* s, const plk_mok_problem* p, int pass, void* stream) {
+  const plk_mok::Dims d = dims_of(p, pass);
+  int rc = PLK_OK;
+  if (plk_mok::workspace_words(d) > s->workspace_words) {
+    // a larger problem than any before: the launches that use the present workspace end first
+    if (stream_is_capturing(stream))
+      return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_forward: this problem needs a larger workspace; run the forward once "
+                                               "before capturing it into a graph");
+    rc = plk_hip_synchronize(nullptr);
+    if (rc == PLK_OK) rc = make_workspace(s, plk_mok::workspace_words(d));
+    if (rc != PLK_OK) return rc;
+  }
+  std::vector<unsigned char> image(s->link.params_bytes, 0);
+  fill_image(s->link, p, pass, s->workspace, image.data());
+  if (image != s->params_host[pass]) {
+    // a new problem: its params image goes to the device first, which synchronises and cannot be part of a graph
+    if (stream_is_capturing(stream))
+      return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_forward: this problem's params image is not on the device yet; run the "
+                                               "forward once before capturing it into a graph");
+    rc = plk_hip_upload(s->params_dev[pass], image.data(), image.size(), stream);
+    if (rc != PLK_OK) return rc;
+    s->params_host[pass].swap(image);
+  }
+  return launch_pass(s, p, pass, stream, s->params_dev[pass]);
 }
 
 int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass, void* stream) {
@@ -176,26 +240,34 @@ int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass,
   int rc = check_problem(p);
   if (rc != PLK_OK) return rc;
   if (p->routed_rows == 0) return PLK_OK;  // nothing routed to this rank
-
-  const int slot = pass - 1;
-  std::vector<unsigned char> image(s->link.params_bytes, 0);
-  fill_image(s->link, p, pass, image.data());
-  if (image != s->params_host[slot]) {
-    // a new problem: its params image goes to the device first, which synchronises and cannot be part of a graph
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (stream && hipStreamIsCapturing((hipStream_t)stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusActive)
-      return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_forward: this problem's params image is not on the device yet; run the "
-                                               "forward once before capturing it into a graph");
-    rc = plk_hip_upload(s->params_dev[slot], image.data(), image.size(), stream);
-    if (rc != PLK_OK) return rc;
-    s->params_host[slot].swap(image);
-  }
-  return launch_pass(s, p, pass, stream, s->params_dev[slot]);
+  return forward_launch(s, p, pass, stream);
 }
 
 int plk_mok_forward(plk_mok_session* s, const plk_mok_problem* p, void* stream) {
-  int rc = plk_mok_forward_pass(s, p, 1, stream);
-  if (rc == PLK_OK) rc = plk_mok_forward_pass(s, p, 2, stream);
+  if (!s) return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok_forward: null session");
+  int rc = check_problem(p);
+  if (rc != PLK_OK) return rc;
+  if (p->routed_rows == 0) return PLK_OK;
+  if (plk_mok::one_launch_ok(dims_of(p, 0), p->hidden_q)) return forward_launch(s, p, 0, stream);
+  rc = forward_launch(s, p, 1, stream);  // rows of `hidden` that share cache lines: the launch boundary orders the two GEMMs
+  if (rc == PLK_OK) rc = forward_launch(s, p, 2, stream);
+  return rc;
+}
+
+int plk_mok_status(plk_mok_session* s, void* stream, uint32_t* status) {
+  if (!s || !status) return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok_status: null argument");
+  uint32_t word = 0;
+  int rc = plk_hip_readback(&word, s->workspace + MOK_WS_STATUS * 4, sizeof word, stream);  // waits for the stream
+  if (rc != PLK_OK) return rc;
+  if (word) rc = plk_hip_zero(s->workspace + MOK_WS_STATUS * 4, sizeof word, stream);
+  if (rc == PLK_OK && s->used_static && g_static_area[s->device]) {
+    const uint64_t at = (uint64_t)(uintptr_t)(g_static_area[s->device] + STATIC_WORKSPACE_OFFSET) + MOK_WS_STATUS * 4;
+    uint32_t other = 0;
+    rc = plk_hip_readback(&other, at, sizeof other, stream);
+    if (rc == PLK_OK && other) rc = plk_hip_zero(at, sizeof other, stream);
+    word |= other;
+  }
+  *status = word;
   return rc;
 }
 
@@ -205,25 +277,35 @@ int plk_mok_forward_static(plk_mok_session* s, const plk_mok_problem* p, void* s
   if (rc != PLK_OK) return rc;
   if (s->link.params_bytes > PLK_MOK_STATIC_IMAGE_BYTES)
     return plk_hip_set_error(PLK_E_CAPACITY, "plk_mok_forward_static: the linked image's params exceed "
-                                             "PLK_MOK_STATIC_IMAGE_BYTES (1024) per pass");
+                                             "PLK_MOK_STATIC_IMAGE_BYTES (1024) per launch");
+  const int64_t words = plk_mok::workspace_words(dims_of(p, 0));
+  if (words > PLK_MOK_STATIC_WORKSPACE_WORDS)
+    return plk_hip_set_error(PLK_E_CAPACITY, "plk_mok_forward_static: routed_rows / 256 + num_experts + 32 exceeds "
+                                             "PLK_MOK_STATIC_WORKSPACE_WORDS (16384)");
   if (p->routed_rows == 0) return PLK_OK;
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev != s->device)
     return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok_forward_static: the session's device must be the current one");
   unsigned char* const base = g_static_area[dev];  // resolved when the session was created on this device
   if (!base) return plk_hip_set_error(PLK_E_RESOURCE, "plk_mok_forward_static: the device's static area was not resolved");
+  const uint64_t workspace = (uint64_t)(uintptr_t)(base + STATIC_WORKSPACE_OFFSET);
 
-  // Both passes' params images travel as the argument of a small kernel that stores them into the static area:
-  // no copy from host memory, no wait, and stream order puts it in front of the two launches that read it.
+  // The launches' params images travel as the argument of a small kernel that stores them into the static area and
+  // clears the workspace: no copy from host memory, no wait, and stream order puts it in front of the launches.
+  const bool one = plk_mok::one_launch_ok(dims_of(p, 0), p->hidden_q);
+  const int passes[2] = {one ? 0 : 1, 2};
+  const int launches = one ? 1 : 2;
   StaticImages images;
   std::memset(&images, 0, sizeof images);
-  for (int pass = 1; pass <= 2; ++pass)
-    fill_image(s->link, p, pass, reinterpret_cast<unsigned char*>(images.words) + (pass - 1) * PLK_MOK_STATIC_IMAGE_BYTES);
-  plk_mok_store_images<<<dim3(1), dim3(STATIC_WORDS), 0, (hipStream_t)stream>>>(images, reinterpret_cast<uint32_t*>(base));
+  for (int l = 0; l < launches; ++l)
+    fill_image(s->link, p, passes[l], workspace, reinterpret_cast<unsigned char*>(images.words) + l * PLK_MOK_STATIC_IMAGE_BYTES);
+  plk_mok_store_images<<<dim3(1), dim3(STATIC_IMAGE_WORDS), 0, (hipStream_t)stream>>>(
+      images, reinterpret_cast<uint32_t*>(base), reinterpret_cast<uint32_t*>(base + STATIC_WORKSPACE_OFFSET), (int)words);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return plk_hip_set_error(PLK_E_RESOURCE, hipGetErrorString(e));
-  for (int pass = 1; pass <= 2 && rc == PLK_OK; ++pass)
-    rc = launch_pass(s, p, pass, stream, (uint64_t)(uintptr_t)(base + (pass - 1) * PLK_MOK_STATIC_IMAGE_BYTES));
+  s->used_static = true;
+  for (int l = 0; l < launches && rc == PLK_OK; ++l)
+    rc = launch_pass(s, p, passes[l], stream, (uint64_t)(uintptr_t)(base + l * PLK_MOK_STATIC_IMAGE_BYTES));
   return rc;
 }
 

@@ -94,7 +94,7 @@ std::vector<Layout> inventory(const char* owner) {
   } else if (!std::strcmp(owner, "mok_act")) {
     v.push_back(L(MOK_ABI_TYPE_ID_MokActResidue, MokActResidue, M(MokActResidue, hidden_q) + M(MokActResidue, hidden_sc) + M(MokActResidue, rows) + M(MokActResidue, cols) + M(MokActResidue, ld_q) + M(MokActResidue, ld_sc) + M(MokActResidue, swiglu_limit) + M(MokActResidue, reserved)));
   } else {
-    v.push_back(L(MOK_ABI_TYPE_ID_MokFrameworkParams, MokFrameworkParams, M(MokFrameworkParams, tokens_per_expert) + M(MokFrameworkParams, expert_row_begin) + M(MokFrameworkParams, expert_tile_begin) + M(MokFrameworkParams, num_experts) + M(MokFrameworkParams, op) + M(MokFrameworkParams, num_col_tiles) + M(MokFrameworkParams, reserved)));
+    v.push_back(L(MOK_ABI_TYPE_ID_MokFrameworkParams, MokFrameworkParams, M(MokFrameworkParams, tokens_per_expert) + M(MokFrameworkParams, workspace) + M(MokFrameworkParams, num_experts) + M(MokFrameworkParams, op) + M(MokFrameworkParams, num_col_tiles_gate_up) + M(MokFrameworkParams, num_col_tiles_down)));
   }
   return v;
 }
@@ -124,7 +124,7 @@ bool read_dims(const plk_shared_scalars_v2* shared, plk_mok::Dims& d) {
   if (!shared || shared->header.abi_version != PLK_HOST_ABI_V2 || shared->header.struct_bytes != sizeof(*shared)) return false;
   if ((uint64_t)shared->record_offset + (uint64_t)shared->record_count * sizeof(plk_scalar_v2) > shared->image_bytes) return false;
   const auto* rec = reinterpret_cast<const plk_scalar_v2*>(reinterpret_cast<const unsigned char*>(shared) + shared->record_offset);
-  int64_t v[65] = {};
+  int64_t v[66] = {};
   uint64_t seen = 0;
   double limit = 0;
   bool have_limit = false;
@@ -136,16 +136,16 @@ bool read_dims(const plk_shared_scalars_v2* shared, plk_mok::Dims& d) {
       have_limit = true;
       continue;
     }
-    const bool known = (id >= 1 && id <= 4) || id == MOK_SCALAR_PASS || id == MOK_SCALAR_PRECISION || (id >= 60 && id <= 64);
+    const bool known = (id >= 1 && id <= 4) || id == MOK_SCALAR_PASS || id == MOK_SCALAR_PRECISION || (id >= 60 && id <= 65);
     if (!known) continue;  // other owners' scalars
     if (rec[i].scalar_type != PLK_SCALAR_I64) return false;
     std::memcpy(&v[id], &rec[i].value_bits, 8);
     if (v[id] < 0 || v[id] > INT32_MAX) return false;
-    seen |= 1ull << (id >= 60 ? id - 40 : id);  // ids 60..64 -> bits 20..24
+    seen |= 1ull << (id >= 60 ? id - 40 : id);  // ids 60..65 -> bits 20..25
   }
-  for (uint32_t id : {1u, 2u, 3u, 4u, 11u, 12u, 60u, 61u, 62u, 63u, 64u})
+  for (uint32_t id : {1u, 2u, 3u, 4u, 11u, 12u, 60u, 61u, 62u, 63u, 64u, 65u})
     if (!(seen & (1ull << (id >= 60 ? id - 40 : id)))) return false;
-  if (!have_limit || v[MOK_SCALAR_PRECISION] != 1 || (v[MOK_SCALAR_PASS] != 1 && v[MOK_SCALAR_PASS] != 2)) return false;
+  if (!have_limit || v[MOK_SCALAR_PRECISION] != 1 || v[MOK_SCALAR_PASS] < 0 || v[MOK_SCALAR_PASS] > 2) return false;
   d.tokens = (int32_t)v[MOK_SCALAR_NUM_LOCAL_TOKENS];
   d.hidden = (int32_t)v[MOK_SCALAR_HIDDEN];
   d.intermediate = (int32_t)v[MOK_SCALAR_INTERMEDIATE];
@@ -157,6 +157,8 @@ bool read_dims(const plk_shared_scalars_v2* shared, plk_mok::Dims& d) {
   d.ld_sc_i = (int32_t)v[MOK_SCALAR_LD_SC_I];
   d.pass = (int32_t)v[MOK_SCALAR_PASS];
   d.swiglu_limit = (float)limit;
+  if (v[MOK_SCALAR_WORKSPACE_WORDS] != plk_mok::workspace_words(d)) return false;
+  if (d.pass == 0 && d.ld_q_i % 128) return false;  // one launch for both GEMMs wants whole cache lines per row of `hidden`
   return plk_mok::check_dims(d) == nullptr;
 }
 
@@ -187,6 +189,8 @@ Shape channel_shape(const char* owner, uint32_t id, const plk_mok::Dims& d) {
     }
   } else if (id == 1) {
     return {1, 32, PLK_ACCESS_READ, {E}};
+  } else if (id == 2) {
+    return {1, 32, PLK_ACCESS_WRITE, {(uint64_t)plk_mok::workspace_words(d)}};
   }
   return {};
 }
@@ -281,6 +285,7 @@ int build(const char* owner, const plk_common_v2* common, const void* args, cons
   }
   std::memset(residue, 0, need);
   if (gemm) {
+    if (d.pass == 0 && !plk_mok::one_launch_ok(d, addr[8])) return PLK_E_RESOURCE;  // hidden_q rows must be whole cache lines
     plk_mok::GemmAddresses a{addr[0], addr[1], addr[2], addr[3], addr[4], addr[5], addr[6], addr[7], addr[8], addr[9], addr[10], addr[11]};
     const MokGemmResidue g = plk_mok::gemm_residue(d, a);
     std::memcpy(residue, &g, sizeof g);
@@ -288,7 +293,7 @@ int build(const char* owner, const plk_common_v2* common, const void* args, cons
     const MokActResidue a = plk_mok::act_residue(d, addr[0], addr[1]);
     std::memcpy(residue, &a, sizeof a);
   } else {
-    const MokFrameworkParams f = plk_mok::framework_params(d, addr[0]);
+    const MokFrameworkParams f = plk_mok::framework_params(d, addr[0], addr[1]);
     std::memcpy(residue, &f, sizeof f);
   }
   return PLK_OK;

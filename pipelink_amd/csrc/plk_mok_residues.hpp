@@ -22,7 +22,7 @@ struct Dims {
   int32_t tokens = 0, hidden = 0, intermediate = 0, experts = 0, routed_rows = 0;
   int32_t ld_q_h = 0, ld_q_i = 0;    // code row pitch of x / hidden, bytes
   int32_t ld_sc_h = 0, ld_sc_i = 0;  // scale row pitch of x / hidden
-  int32_t pass = 1;                  // 1 = gate/up + SwiGLU + requant, 2 = down
+  int32_t pass = 0;                  // 0 = both GEMMs in one launch, 1 = gate/up + SwiGLU + requant, 2 = down
   float swiglu_limit = 7.0f;
 };
 
@@ -89,23 +89,34 @@ inline MokActResidue act_residue(const Dims& d, uint64_t hidden_q, uint64_t hidd
   return a;
 }
 
-inline int32_t num_col_tiles(const Dims& d) {
-  return d.pass == 1 ? (d.intermediate + TILE_W / 2 - 1) / (TILE_W / 2) : (d.hidden + TILE_W - 1) / TILE_W;
-}
+inline int32_t num_col_tiles_gate_up(const Dims& d) { return (d.intermediate + TILE_W / 2 - 1) / (TILE_W / 2); }
+inline int32_t num_col_tiles_down(const Dims& d) { return (d.hidden + TILE_W - 1) / TILE_W; }
 
-inline MokFrameworkParams framework_params(const Dims& d, uint64_t tokens_per_expert) {
+// an upper bound of the number of routed-row tiles: every expert may end in a partial tile
+inline int64_t max_row_tiles(const Dims& d) { return ((int64_t)d.routed_rows + TILE_X - 1) / TILE_X + d.experts; }
+
+// 32-bit words of the launch workspace (MOK_WS_* words, then one readiness counter per routed-row tile)
+inline int64_t workspace_words(const Dims& d) { return MOK_WS_COUNTERS + max_row_tiles(d); }
+
+// One launch may run both GEMMs only if no cache line of `hidden` is shared between two gate/up tiles, whose
+// workgroups may sit on different XCDs: rows that start and end on 128-byte boundaries (a gate/up tile writes 128
+// bytes of a row).  Otherwise the forward is two launches.
+inline bool one_launch_ok(const Dims& d, uint64_t hidden_q) { return d.ld_q_i % 128 == 0 && hidden_q % 128 == 0; }
+
+inline MokFrameworkParams framework_params(const Dims& d, uint64_t tokens_per_expert, uint64_t workspace) {
   MokFrameworkParams fw{};
   fw.tokens_per_expert = (const int32_t*)(uintptr_t)tokens_per_expert;
+  fw.workspace = (uint32_t*)(uintptr_t)workspace;
   fw.num_experts = d.experts;
-  fw.op = d.pass == 1 ? MOK_GEMM_FWD_ROUTED_GATE_UP : MOK_GEMM_FWD_ROUTED_DOWN;
-  fw.num_col_tiles = num_col_tiles(d);
+  fw.op = d.pass == 0 ? MOK_FWD_BOTH : d.pass == 1 ? MOK_GEMM_FWD_ROUTED_GATE_UP : MOK_GEMM_FWD_ROUTED_DOWN;
+  fw.num_col_tiles_gate_up = num_col_tiles_gate_up(d);
+  fw.num_col_tiles_down = num_col_tiles_down(d);
   return fw;
 }
 
-// an upper bound of the number of tiles of one pass: more workgroups than this would idle
+// an upper bound of the number of tiles of the launch: more workgroups than this would idle
 inline int64_t max_workgroups(const Dims& d) {
-  const int64_t max_row_tiles = ((int64_t)d.routed_rows + TILE_X - 1) / TILE_X + d.experts;
-  return max_row_tiles * num_col_tiles(d);
+  return max_row_tiles(d) * ((d.pass != 2 ? num_col_tiles_gate_up(d) : 0) + (d.pass != 1 ? num_col_tiles_down(d) : 0));
 }
 
 }  // namespace plk_mok

@@ -154,9 +154,9 @@ class MokActResidue(Structure):
 
 
 class MokFrameworkParams(Structure):
-    _fields_ = [("tokens_per_expert", c_void_p), ("expert_row_begin", c_void_p), ("expert_tile_begin", c_void_p),
-                ("num_experts", ctypes.c_int32), ("op", ctypes.c_int32), ("num_col_tiles", ctypes.c_int32),
-                ("reserved", ctypes.c_int32)]
+    _fields_ = [("tokens_per_expert", c_void_p), ("workspace", c_void_p),
+                ("num_experts", ctypes.c_int32), ("op", ctypes.c_int32), ("num_col_tiles_gate_up", ctypes.c_int32),
+                ("num_col_tiles_down", ctypes.c_int32)]
 
 
 # neutral inventory, in the order the providers report it (type id, C name, mirror)

@@ -130,6 +130,14 @@ class MoKSession:
                           w_up_sc=w_up_sc.data_ptr(), w_down_q=w_down_q.data_ptr(), w_down_sc=w_down_sc.data_ptr(),
                           hidden_q=hidden_q.data_ptr(), hidden_sc=hidden_sc.data_ptr(), y=y.data_ptr())
 
+    def status(self, stream: int | None = None) -> int:
+        """Waits for the stream, then returns and clears the launches' sticky status word (``plk_mok_status``): 0, or
+        bit 0 = a dependency wait inside a one-launch forward gave up."""
+        s = c_void_p(torch.cuda.current_stream().cuda_stream if stream is None else stream)
+        word = ctypes.c_uint32(0)
+        check(self.lib, self.lib.plk_mok_status(self._handle, s, byref(word)))
+        return word.value
+
     def forward_static(self, problem: MokProblem, stream: int | None = None) -> None:
         """Both passes through the entry point that allocates nothing (``plk_mok_forward_static``): the params images
         go into a fixed area of device memory the library owns; calls that overlap on one GPU race on it."""
@@ -137,7 +145,8 @@ class MoKSession:
         check(self.lib, self.lib.plk_mok_forward_static(self._handle, byref(problem), s))
 
     def forward(self, problem: MokProblem, stream: int | None = None, which: int = 0) -> None:
-        """Launch both passes (``which=0``) or one of them (1 = gate/up+SwiGLU+requant, 2 = down)."""
+        """The whole forward (``which=0``: one launch when hidden_q's rows are whole 128-byte lines, else two) or one
+        pass of it (1 = gate/up+SwiGLU+requant, 2 = down)."""
         s = c_void_p(torch.cuda.current_stream().cuda_stream if stream is None else stream)
         if which == 0:
             check(self.lib, self.lib.plk_mok_forward(self._handle, byref(problem), s))

@@ -41,14 +41,23 @@ def route(logits: torch.Tensor, top_k: int):
 
 
 def generate(num_tokens: int, hidden: int, intermediate: int, num_experts: int, top_k: int, seed: int = 0,
-             concentrate: int = 0, quantize_device: torch.device | None = None) -> MokInputs:
-    """``concentrate`` > 0 routes every token to the first ``concentrate`` experts only (empty experts)."""
+             concentrate: int = 0, quantize_device: torch.device | None = None,
+             counts: list[int] | None = None) -> MokInputs:
+    """``concentrate`` > 0 routes every token to the first ``concentrate`` experts only (empty experts).
+    ``counts`` sets the experts' row counts directly (``top_k`` is then unused): every routed row reads a token
+    drawn at random."""
     g = torch.Generator().manual_seed(seed)
     logits = torch.randn(num_tokens, num_experts, generator=g)
     if concentrate:
         logits[:, concentrate:] = -1e9
     x = torch.randn(num_tokens, hidden, generator=g)
-    counts, row_token = route(logits, top_k)
+    if counts is not None:
+        if len(counts) != num_experts:
+            raise ValueError("counts must give one row count per expert")
+        row_token = torch.randint(num_tokens, (sum(counts),), generator=g).to(torch.int32)
+        counts = torch.tensor(counts, dtype=torch.int32)
+    else:
+        counts, row_token = route(logits, top_k)
     dev = quantize_device or torch.device("cpu")
     x_q, x_sc = mxfp8.quantize(x.to(dev))
 

@@ -39,6 +39,9 @@ __device__ __forceinline__ float min_raw(float a, float b) {
 
 template <bool CLAMPED>
 __device__ __forceinline__ float swiglu(float gate, float up, float limit) {
+#ifdef EXP_NOEPI
+  return gate + up;
+#endif
   if (CLAMPED) {
     gate = min_raw(gate, limit);
     up = __builtin_amdgcn_fmed3f(up, -limit, limit);
@@ -50,6 +53,7 @@ __device__ __forceinline__ float swiglu(float gate, float up, float limit) {
 }
 
 typedef short s16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((__vector_size__(16)));
 
 // Four floats -> four e4m3 codes of a block whose scale is `scale` (a power of two): round to
 // bf16 (nearest even, v_cvt_pk_bf16_f32: the reference rounds to bf16 before quantising,
@@ -68,7 +72,7 @@ __device__ __forceinline__ uint32_t quantise4(float a, float b, float c, float d
 }
 
 template <bool CLAMPED>
-__device__ __forceinline__ void forward(const MokActResidue& p, const MokActTask& t, const AccFrag& acc) {
+__device__ __forceinline__ void forward(const MokActResidue& p, const MokActTask& t, const AccFrag& acc, const MokCounters& counters) {
   const int tid = fresh_tid();
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -112,15 +116,20 @@ __device__ __forceinline__ void forward(const MokActResidue& p, const MokActTask
   }
   __syncthreads();
   // ---- coalesced write-out: a row is 128 bytes = 8 lanes x 16 bytes, 8 rows per wave store ----
+  // Stores of `hidden` are device-scope (cache policy bit 4, sc1): they go through to memory, where a workgroup on
+  // another XCD -- a down tile of the same launch, once the row tile's counter says so -- reads them.
   const int chunk = lane & 7;
   const bool col_ok = t.col_begin + chunk * 16 < p.cols;  // column extents are multiples of 32
+  const __amdgpu_buffer_rsrc_t out_q =
+      __builtin_amdgcn_make_buffer_rsrc(p.hidden_q, 0, (int)((uint32_t)p.rows * (uint32_t)p.ld_q), 0x00020000);
 #pragma unroll
   for (int it = 0; it < TILE_X / (THREADS / 64) / 8; ++it) {
     const int trow = wave * (TILE_X / (THREADS / 64)) + it * 8 + (lane >> 3);
     const int row = t.row_begin + trow;
     if (row < t.row_end && col_ok) {
-      const uint4 v = *reinterpret_cast<const uint4*>(stage + trow * STAGE_PITCH + chunk * 16);
-      *reinterpret_cast<uint4*>(p.hidden_q + (int64_t)row * p.ld_q + t.col_begin + chunk * 16) = v;
+      const v4i v = *reinterpret_cast<const v4i*>(stage + trow * STAGE_PITCH + chunk * 16);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), out_q,
+                                             (int)((uint32_t)row * (uint32_t)p.ld_q + (uint32_t)(t.col_begin + chunk * 16)), 0, 16);
     }
   }
   static_assert(THREADS == TILE_X, "one thread per routed row writes the row's scale bytes");
@@ -130,13 +139,20 @@ __device__ __forceinline__ void forward(const MokActResidue& p, const MokActTask
       const uint32_t sc = *reinterpret_cast<const uint32_t*>(stage + STAGE_SCALE_OFF + tid * 4);
       uint8_t* out = p.hidden_sc + (int64_t)row * p.ld_sc + (t.col_begin >> 5);
       if (t.col_begin + TILE_W / 2 <= p.cols) {
-        *reinterpret_cast<uint32_t*>(out) = sc;  // col_begin is a multiple of 128: dword aligned
+        // col_begin is a multiple of 128: dword aligned
+        __hip_atomic_store(reinterpret_cast<uint32_t*>(out), sc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       } else {
-        for (int j = 0; t.col_begin + 32 * j < p.cols; ++j) out[j] = (uint8_t)(sc >> (8 * j));
+        for (int j = 0; t.col_begin + 32 * j < p.cols; ++j)
+          __hip_atomic_store(out + j, (uint8_t)(sc >> (8 * j)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
   }
-  __syncthreads();  // the staging tile shares LDS with the GEMM ring of the next tile
+  // Every wave's stores have completed (the barrier's fence waits for them) before the tile is counted: the row tile's
+  // counter reaches the number of gate/up column tiles when all of its `hidden` is in memory
+  // (campaigns/mok/port/framework/interp_fwd.cu:174-213: the reference's act -> down dependency).
+  __syncthreads();  // also: the staging tile shares LDS with the GEMM ring of the next tile
+  if (t.counter_idx >= 0 && counters.base && tid == 0)
+    __hip_atomic_fetch_add(counters.base + t.counter_idx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace mok_act_owner
@@ -145,13 +161,12 @@ extern "C" __device__ void mok_act_init(const void* view) { (void)view; }
 
 extern "C" __device__ void mok_act_fwd(const void* view, const MokActTask* task, const MokCounters* counters,
                                        uint32_t* phase, const mok::AccFrag* acc) {
-  (void)counters;
   (void)phase;
   const auto& p = *static_cast<const MokActResidue*>(static_cast<const pipelink_host_view*>(view)->residue);
   if (pipelink_mok_clamp())
-    mok_act_owner::forward<true>(p, *task, *acc);
+    mok_act_owner::forward<true>(p, *task, *acc, *counters);
   else
-    mok_act_owner::forward<false>(p, *task, *acc);
+    mok_act_owner::forward<false>(p, *task, *acc, *counters);
 }
 #else  // PIPELINK_EMIT: host-evaluated annotations only
 #include "../include/mok_abi.h"

@@ -4,12 +4,24 @@
 // published facts TILE_X / TILE_W.
 //
 // Plays the part of mok_framework_run in campaigns/mok/port/framework/interp_fwd.cu:26-252
-// (task decode :137-214).  Not carried over: CLC work stealing and 2-CTA clusters (no
-// gfx950 counterpart) and the comm clusters (single GPU).  The schedule here is static:
-// tiles are numbered expert-major, within one expert column-tile-major with the row tiles
-// innermost, so workgroups that run at the same time share one weight tile; the tile
-// range is split in 8 contiguous chunks, one per XCD (workgroup id % 8), so each L2 sees
-// a contiguous run of experts.
+// (task decode :137-214, dependency chain gate/up -> act -> down :174-213).  Not carried over: 2-CTA clusters (no
+// gfx950 counterpart) and the comm clusters (single GPU).
+//
+// One launch runs both GEMMs (op MOK_FWD_BOTH) or one of them.  The tiles are in eight lists, one per XCD (workgroup
+// id % 8): list q holds the tiles of an eighth of the routed-row tiles -- the gate/up tiles first, then the down tiles
+// of the same rows; within each, expert by expert, column tile by column tile, row tiles innermost, so that
+// workgroups that run at the same time share a weight tile and one XCD's L2 sees a contiguous run of experts.  The
+// schedule is static: the workgroups of an XCD take the items of its list in turn (the reference asks the cluster
+// launch control for its next tile, interp_fwd.cu:137-160; tiles of one size gain nothing from that here, and a
+// static turn costs no atomic and no barrier).  A down tile reads rows of `hidden` that up to 23 other workgroups
+// write: it waits until the row tile's readiness counter (MokCounters) has reached the number of gate/up column
+// tiles.  Every workgroup runs all its gate/up tiles before its first down tile, gate/up tiles wait for nothing, and
+// a workgroup only ever waits while it holds no unfinished tile: so the tiles a wait depends on are finished or
+// running, no wait can last, and each is bounded anyway.
+//
+// Per workgroup the tiles are software-pipelined: the next tile's row tokens and readiness counter are requested
+// behind the current tile's first loads (mok_gemm_fwd's `upcoming`), and its first loads are issued between the
+// current tile's mainloop and epilogue.
 #include <pipelink/stage.hpp>
 #ifndef PIPELINK_EMIT
 #include "../include/mok_device.hpp"
@@ -17,10 +29,14 @@
 extern "C" __device__ int pipelink_mok_fw_sched();  // byte offset of the schedule table in dynamic LDS
 
 extern "C" __device__ void pipelink_call_gemm_init(const void* view);
+extern "C" __device__ void pipelink_call_gemm_fini(const void* view);
 extern "C" __device__ void pipelink_call_act_init(const void* view);
+extern "C" __device__ void pipelink_call_gemm_stage(const void* view, const MokGemmTask*, const MokCounters*);
+extern "C" __device__ bool pipelink_call_gemm_ready(const void* view, const MokGemmTask*, const MokCounters*);
+extern "C" __device__ void pipelink_call_gemm_wait(const void* view, const MokGemmTask*, const MokCounters*);
 extern "C" __device__ void pipelink_call_gemm_prefetch(const void* view, const MokGemmTask*, mok::GemmCarry*);
 extern "C" __device__ void pipelink_call_gemm_fwd(const void* view, const MokGemmTask*, const MokCounters*, uint32_t*,
-                                                  mok::AccFrag*, const mok::GemmCarry*);
+                                                  mok::AccFrag*, const mok::GemmCarry*, const MokGemmTask*);
 extern "C" __device__ void pipelink_call_gemm_store(const void* view, const MokGemmTask*, const mok::AccFrag*);
 extern "C" __device__ void pipelink_call_act_fwd(const void* view, const MokActTask*, const MokCounters*, uint32_t*,
                                                  const mok::AccFrag*);
@@ -29,16 +45,72 @@ extern __shared__ __attribute__((aligned(1024))) unsigned char pipelink_smem[];
 
 namespace mok_framework {
 constexpr int MAX_EXPERTS = 256;
-constexpr int NUM_XCD = 8;
-}
+constexpr int NUM_XCD = 8;       // lists
+
+// the schedule's tables in LDS: exclusive prefix sums per expert, and one word of the last workgroup
+struct Tables {
+  int row_begin[MAX_EXPERTS + 1];
+  int tile_begin[MAX_EXPERTS + 1];
+  uint32_t last;  // 1 in the workgroup that leaves the launch last
+};
+
+struct Schedule {
+  const MokFrameworkParams& g;
+  const Tables& tab;
+  int row_tiles;  // of all experts
+  int gate_up_cols, down_cols;  // column tiles of the GEMMs this launch runs (0: not run)
+
+  // List q: the q-th eighth of the gate/up tiles (all experts' tiles in one sequence: expert by expert, column tile by
+  // column tile, row tiles innermost), then the q-th eighth of the down tiles.
+  __device__ __forceinline__ int share(int q, int total) const { return (int)((long long)q * total / NUM_XCD); }
+  __device__ __forceinline__ int length(int q) const {
+    const int gu = row_tiles * gate_up_cols, d = row_tiles * down_cols;
+    return share(q + 1, gu) - share(q, gu) + share(q + 1, d) - share(q, d);
+  }
+
+  // item i of list q -> task.  `cursor` is the expert of the item this workgroup decoded last: a workgroup's items
+  // come in growing order as long as it stays in one GEMM, so the search usually ends where it starts.
+  __device__ __forceinline__ MokGemmTask decode(int q, int i, int& cursor) const {
+    const int gu = row_tiles * gate_up_cols, d = row_tiles * down_cols;
+    const int gate_up_items = share(q + 1, gu) - share(q, gu);
+    const bool gate_up = i < gate_up_items;
+    const int idx = gate_up ? share(q, gu) + i : share(q, d) + i - gate_up_items;  // in the sequence of its GEMM's tiles
+    const int cols = gate_up ? gate_up_cols : down_cols;
+    // last e with tile_begin[e] * cols <= idx: it has row tiles, since tile_begin[e + 1] * cols > idx
+    int lo = cursor;
+    if (tab.tile_begin[lo] * cols > idx) lo = 0;  // the other GEMM: from the start
+    while (lo + 1 < g.num_experts && tab.tile_begin[lo + 1] * cols <= idx) ++lo;
+    cursor = lo;
+    const int e = __builtin_amdgcn_readfirstlane(lo);
+    const int t0 = tab.tile_begin[e], t1 = tab.tile_begin[e + 1];
+    const int local = idx - t0 * cols;
+    const int col = local / (t1 - t0);
+    const int tile = t0 + local - col * (t1 - t0);  // row tile, counted over all experts
+    const int first = tab.row_begin[e] + (tile - tab.tile_begin[e]) * mok::TILE_X;
+    const bool both = g.op == MOK_FWD_BOTH;
+    // wave-uniform by construction; say so, so that the task lives in scalar registers
+    MokGemmTask t;
+    t.op = gate_up ? MOK_GEMM_FWD_ROUTED_GATE_UP : MOK_GEMM_FWD_ROUTED_DOWN;
+    t.expert = e;
+    t.row_begin = __builtin_amdgcn_readfirstlane(first);
+    t.row_end = __builtin_amdgcn_readfirstlane(tab.row_begin[e + 1]);
+    t.col_begin = __builtin_amdgcn_readfirstlane(col * (gate_up ? mok::TILE_W / 2 : mok::TILE_W));
+    t.task_idx = __builtin_amdgcn_readfirstlane(q << 24 | i);
+    t.counter_idx = __builtin_amdgcn_readfirstlane(both ? tile : -1);
+    t.wait_target = gate_up ? 0 : gate_up_cols;
+    t.flags = 0u;
+    return t;
+  }
+};
+
+}  // namespace mok_framework
 
 extern "C" __device__ void mok_framework_worker(const void* params, unsigned variant) {
   (void)variant;
   using namespace mok_framework;
   const pipelink_host_view view{params, nullptr};
   const MokFrameworkParams& g = *static_cast<const MokFrameworkParams*>(params);
-  int* row_begin = reinterpret_cast<int*>(pipelink_smem + pipelink_mok_fw_sched());
-  int* tile_begin = row_begin + (MAX_EXPERTS + 1);
+  Tables& tab = *reinterpret_cast<Tables*>(pipelink_smem + pipelink_mok_fw_sched());
   const int ne = g.num_experts;
 
   pipelink_call_gemm_init(&view);
@@ -48,101 +120,145 @@ extern "C" __device__ void mok_framework_worker(const void* params, unsigned var
   if (threadIdx.x == 0) {
     int rows = 0, tiles = 0;
     for (int e = 0; e < ne; ++e) {
-      row_begin[e] = rows;
-      tile_begin[e] = tiles;
+      tab.row_begin[e] = rows;
+      tab.tile_begin[e] = tiles;
       const int c = g.tokens_per_expert[e];
       rows += c;
       tiles += (c + mok::TILE_X - 1) / mok::TILE_X;
     }
-    row_begin[ne] = rows;
-    tile_begin[ne] = tiles;
+    tab.row_begin[ne] = rows;
+    tab.tile_begin[ne] = tiles;
   }
   __syncthreads();
 
-  const int nct = g.num_col_tiles;
-  const int total = tile_begin[ne] * nct;
-  const int chunk = (total + NUM_XCD - 1) / NUM_XCD;
-  const int xcd = blockIdx.x % NUM_XCD;
-  const int per_xcd = gridDim.x / NUM_XCD;  // launch grid is a multiple of NUM_XCD
-  const int chunk_end = min(total, (xcd + 1) * chunk);
-  const MokCounters counters{nullptr};
+  const Schedule sched{g, tab, tab.tile_begin[ne], g.op == MOK_GEMM_FWD_ROUTED_DOWN ? 0 : g.num_col_tiles_gate_up,
+                       g.op == MOK_GEMM_FWD_ROUTED_GATE_UP ? 0 : g.num_col_tiles_down};
+  const MokCounters counters{g.op == MOK_FWD_BOTH ? reinterpret_cast<int32_t*>(g.workspace + MOK_WS_COUNTERS) : nullptr,
+                             g.workspace + MOK_WS_STATUS};
   uint32_t phase = 0;
 
-  const bool gate_up = g.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
-  auto decode = [&](int idx) {
-    // expert of tile idx: last e with tile_begin[e] * nct <= idx
-    int lo = 0, hi = ne;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (tile_begin[mid] * nct <= idx) lo = mid; else hi = mid;
+  const int q = blockIdx.x % NUM_XCD;
+  const int turn = gridDim.x / NUM_XCD;  // the launch grid is a multiple of NUM_XCD: workgroups per list
+  const int items = sched.length(q);
+  int i = blockIdx.x / NUM_XCD, cursor = 0;
+  if (i < items) {
+    MokGemmTask task = sched.decode(q, i, cursor);
+    // the first tile has no mainloop in front of it to look ahead from
+    pipelink_call_gemm_stage(&view, &task, &counters);
+    __syncthreads();  // waits for the staged loads, then the barrier
+    if (!pipelink_call_gemm_ready(&view, &task, &counters)) pipelink_call_gemm_wait(&view, &task, &counters);
+    mok::GemmCarry carry;
+    pipelink_call_gemm_prefetch(&view, &task, &carry);
+#ifdef EXP_STAMP
+    int exp_tile = 0;
+    const MokGemmResidue* exp_g = reinterpret_cast<const MokGemmResidue*>(static_cast<const unsigned char*>(params) + EXP_STAMP);
+    unsigned long long* exp_stamps = reinterpret_cast<unsigned long long*>(exp_g->y + (size_t)exp_g->hidden.rows * exp_g->ld_y) + (size_t)blockIdx.x * 384;
+    unsigned long long s4 = wall_clock64();
+#endif
+    for (;;) {
+      i += turn;
+      const bool has_next = i < items;
+      MokGemmTask next = task;
+      if (has_next) next = sched.decode(q, i, cursor);
+      else next.op = 0;  // no task: mok_gemm_fwd looks ahead to nothing
+      mok::AccFrag acc;
+#ifdef EXP_STAMP
+      const unsigned long long s0 = wall_clock64();
+#endif
+      pipelink_call_gemm_fwd(&view, &task, &counters, &phase, &acc, &carry, &next);
+#ifdef EXP_STAMP
+      const unsigned long long s1 = wall_clock64();
+#endif
+      // The next tile's first loads fly while this tile's epilogue computes -- unless its rows are not complete yet:
+      // then this tile is finished (and counted) first, so that nobody waits for a workgroup that waits.
+      const bool early = has_next && pipelink_call_gemm_ready(&view, &next, &counters);
+      if (early) pipelink_call_gemm_prefetch(&view, &next, &carry);
+#ifdef EXP_STAMP
+      const unsigned long long s2 = wall_clock64();
+#endif
+      if (task.op == MOK_GEMM_FWD_ROUTED_GATE_UP) {
+        const MokActTask act{MOK_ACT_FWD_ROUTED, task.row_begin, task.row_end, task.col_begin, task.task_idx, task.counter_idx, 0u};
+        pipelink_call_act_fwd(&view, &act, &counters, &phase, &acc);
+      } else {
+        pipelink_call_gemm_store(&view, &task, &acc);
+      }
+#ifdef EXP_STAMP
+      {
+        const unsigned long long s3 = wall_clock64();
+        if (threadIdx.x == 0 && exp_tile < 64) {
+          int rows = task.row_end - task.row_begin; rows = rows > 256 ? 256 : rows;
+          exp_stamps[exp_tile * 6 + 0] = s0; exp_stamps[exp_tile * 6 + 1] = s1; exp_stamps[exp_tile * 6 + 2] = s2;
+          exp_stamps[exp_tile * 6 + 3] = s3; exp_stamps[exp_tile * 6 + 4] = (unsigned)((rows + 31) / 32) | (unsigned)task.op << 8 | (early ? 1u << 16 : 0u);
+          exp_stamps[exp_tile * 6 + 5] = s4;
+        }
+        ++exp_tile;
+        s4 = s3;
+      }
+#endif
+      if (!has_next) break;
+      if (!early) {
+        pipelink_call_gemm_wait(&view, &next, &counters);
+        pipelink_call_gemm_prefetch(&view, &next, &carry);
+      }
+      task = next;
     }
-    const int e = __builtin_amdgcn_readfirstlane(lo);
-    const int mtiles = tile_begin[e + 1] - tile_begin[e];
-    const int local = idx - tile_begin[e] * nct;
-    const int nt = local / mtiles;
-    const int mt = local - nt * mtiles;
-    const int col_begin = nt * (gate_up ? mok::TILE_W / 2 : mok::TILE_W);
-    // wave-uniform by construction; say so, so that the task lives in scalar registers
-    return MokGemmTask{g.op, e, __builtin_amdgcn_readfirstlane(row_begin[e] + mt * mok::TILE_X),
-                       __builtin_amdgcn_readfirstlane(row_begin[e + 1]), __builtin_amdgcn_readfirstlane(col_begin), idx, 0u};
-  };
+  }
+  pipelink_call_gemm_fini(&view);
 
-  // Software pipeline over this workgroup's tiles: the next tile's first loads are issued
-  // between a tile's mainloop and its epilogue, so they fly while the epilogue computes.
-  int idx = xcd * chunk + blockIdx.x / NUM_XCD;
-  if (idx >= chunk_end) return;
-  MokGemmTask task = decode(idx);
-  mok::GemmCarry carry;
-  pipelink_call_gemm_prefetch(&view, &task, &carry);
-  for (;;) {
-    const int next_idx = idx + per_xcd;
-    const bool has_next = next_idx < chunk_end;
-    MokGemmTask next = task;
-    if (has_next) next = decode(next_idx);
-    mok::AccFrag acc;
-    pipelink_call_gemm_fwd(&view, &task, &counters, &phase, &acc, &carry);
-    if (has_next) pipelink_call_gemm_prefetch(&view, &next, &carry);
-    if (gate_up) {
-      const MokActTask act{MOK_ACT_FWD_ROUTED, task.row_begin, task.row_end, task.col_begin, idx, 0u};
-      pipelink_call_act_fwd(&view, &act, &counters, &phase, &acc);
-    } else {
-      pipelink_call_gemm_store(&view, &task, &acc);
-    }
-    if (!has_next) break;
-    task = next;
-    idx = next_idx;
+  // The last workgroup to leave puts the counters back to zero for the next launch: by then nobody waits any more.
+  if (g.op != MOK_FWD_BOTH) return;
+  if (threadIdx.x == 0) {
+    const uint32_t before = __hip_atomic_fetch_add(g.workspace + MOK_WS_FINISHED, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    tab.last = before == gridDim.x - 1 ? 1u : 0u;
+  }
+  __syncthreads();
+  if (tab.last) {
+    for (int w = threadIdx.x; w < sched.row_tiles; w += blockDim.x)
+      __hip_atomic_store(g.workspace + MOK_WS_COUNTERS + w, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) __hip_atomic_store(g.workspace + MOK_WS_FINISHED, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 #else  // PIPELINK_EMIT: host-evaluated annotations only
 #include "../include/mok_abi.h"
 #endif
 
-PL_STAGE("mok.framework", "0.1.0");
+PL_STAGE("mok.framework", "0.2.0");
 PL_PARAMS(MokFrameworkParams);
 PL_ROLE(worker, mok_framework_worker, 4);
 PL_TOPOLOGY(true, "static");
 PL_VARIANT(0, {});
 PL_CALL(gemm_init, "mok_gemm_init", "extern \"C\" __device__ void pipelink_call_gemm_init(const void* view);");
+PL_CALL(gemm_fini, "mok_gemm_fini", "extern \"C\" __device__ void pipelink_call_gemm_fini(const void* view);");
 PL_CALL(act_init, "mok_act_init", "extern \"C\" __device__ void pipelink_call_act_init(const void* view);");
+PL_CALL(gemm_stage, "mok_gemm_stage",
+        "extern \"C\" __device__ void pipelink_call_gemm_stage(const void* view, const MokGemmTask* task, const MokCounters* counters);");
+PL_CALL(gemm_ready, "mok_gemm_ready",
+        "extern \"C\" __device__ bool pipelink_call_gemm_ready(const void* view, const MokGemmTask* task, const MokCounters* counters);");
+PL_CALL(gemm_wait, "mok_gemm_wait",
+        "extern \"C\" __device__ void pipelink_call_gemm_wait(const void* view, const MokGemmTask* task, const MokCounters* counters);");
 PL_CALL(gemm_prefetch, "mok_gemm_prefetch",
         "extern \"C\" __device__ void pipelink_call_gemm_prefetch(const void* view, const MokGemmTask* task, mok::GemmCarry* carry);");
 PL_CALL(gemm_fwd, "mok_gemm_fwd",
         "extern \"C\" __device__ void pipelink_call_gemm_fwd(const void* view, const MokGemmTask* task, "
-        "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc, const mok::GemmCarry* carry);");
+        "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc, const mok::GemmCarry* carry, "
+        "const MokGemmTask* upcoming);");
 PL_CALL(gemm_store, "mok_gemm_store",
         "extern \"C\" __device__ void pipelink_call_gemm_store(const void* view, const MokGemmTask* task, const mok::AccFrag* acc);");
 PL_CALL(act_fwd, "mok_act_fwd",
         "extern \"C\" __device__ void pipelink_call_act_fwd(const void* view, const MokActTask* task, "
         "const MokCounters* counters, uint32_t* phase, const mok::AccFrag* acc);");
-// schedule table: exclusive prefix sums of rows and row tiles for up to 256 experts
-PL_CLAIM("pipelink_mok_fw_sched", "smem", 2 * (256 + 1) * 4, 16, "kernel");
+// schedule tables: exclusive prefix sums of rows and row tiles for up to 256 experts, and one word more
+PL_CLAIM("pipelink_mok_fw_sched", "smem", 2 * (256 + 1) * 4 + 8, 16, "kernel");
 PL_USES("pipelink_mok_fw_sched");
 // host contract: the schedule's owner
 PL_HOST_GROUP("mok.framework.params", "mok_framework");
 PL_HOST_ABI_TYPE(3, MokFrameworkParams);
 MOK_HOST_SCALARS();
 PL_HOST_CHANNEL(1, "tokens_per_expert", 32, "read", "mok.num_local_experts", false);
+// status word and readiness counters of a launch: all zero before the first launch, every launch leaves them zero
+PL_HOST_CHANNEL(2, "workspace", 32, "write", "mok.workspace_words", false);
 PL_FACT("mok.framework.MAX_EXPERTS", 256);
+PL_FACT("mok.framework.LISTS", 8);
 PL_PRELUDE("../include/mok_abi.h");
 PL_PRELUDE("../include/mok_device.hpp");
 PL_EMIT_MAIN()

@@ -70,10 +70,26 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
 }
 // 16 (4) bytes per lane, buffer -> LDS; lane i lands at lds + 16*i (4*i)
 __device__ __forceinline__ void buf16_to_lds(rsrc_t r, uint32_t lane_off, uint32_t uni_off, unsigned char* lds) {
+#ifndef EXP_NOLOADS
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lptr_t)lds, 16, (int)lane_off, (int)uni_off, 0, 0);
+#endif
 }
 __device__ __forceinline__ void buf4_to_lds(rsrc_t r, uint32_t lane_off, uint32_t uni_off, unsigned char* lds) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lptr_t)lds, 4, (int)lane_off, (int)uni_off, 0, 0);
+}
+// The same at device scope (cache policy bit 4, sc1): the load does not trust a line that another XCD's workgroup may
+// have written during this launch.  Used for what one workgroup of the launch writes and another reads where a cache
+// line can hold both finished and unfinished parts: the scale rows of `hidden` (a line spans rows of different row
+// tiles) and the readiness counters.
+__device__ __forceinline__ void buf16_to_lds_device_scope(rsrc_t r, uint32_t lane_off, uint32_t uni_off, unsigned char* lds) {
+#ifdef EXP_NO_SC1_XSC
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lptr_t)lds, 16, (int)lane_off, (int)uni_off, 0, 0);
+#else
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lptr_t)lds, 16, (int)lane_off, (int)uni_off, 0, 16);
+#endif
+}
+__device__ __forceinline__ void buf4_to_lds_device_scope(rsrc_t r, uint32_t lane_off, uint32_t uni_off, unsigned char* lds) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lptr_t)lds, 4, (int)lane_off, (int)uni_off, 0, 16);
 }
 
 struct Loader {
@@ -94,9 +110,11 @@ struct Loader {
 // "head", claimed for the whole kernel) take the next tile's first loads while the current
 // tile's epilogue runs; the other buffers (the "arena", claimed for the GEMM phase only) share
 // their LDS with the epilogue's staging tile.
-//   head : X0 X1 W0 W1 | 4 x 1 KB weight scales | 2 x 4 KB routed-row scales
+//   head : X0 X1 W0 W1 | 4 x 1 KB weight scales | 2 x 4 KB routed-row scales | staged task: 1 KB row tokens, 256 B counter
 //   arena: X2 .. X[DEPTH] | W2 .. W[DEPTH-1]
-constexpr int HEAD_BYTES = 4 * BUF_BYTES + WSCALE_BYTES + XSCALE_BYTES;
+constexpr int STAGED_TOKEN_BYTES = TILE_X * 4;  // row_token of the staged tile's rows
+constexpr int STAGED_PEEK_BYTES = 256;          // one wave's copies of the readiness counter it depends on
+constexpr int HEAD_BYTES = 4 * BUF_BYTES + WSCALE_BYTES + XSCALE_BYTES + STAGED_TOKEN_BYTES + STAGED_PEEK_BYTES;
 template <int DEPTH>
 struct Rings {
   unsigned char* head;
@@ -111,6 +129,8 @@ struct Rings {
   }
   __device__ __forceinline__ unsigned char* wscale() const { return head + 4 * BUF_BYTES; }
   __device__ __forceinline__ unsigned char* xscale() const { return head + 4 * BUF_BYTES + WSCALE_BYTES; }
+  __device__ __forceinline__ unsigned char* tokens() const { return head + 4 * BUF_BYTES + WSCALE_BYTES + XSCALE_BYTES; }
+  __device__ __forceinline__ unsigned char* peek() const { return tokens() + STAGED_TOKEN_BYTES; }
 };
 
 __device__ __forceinline__ int swizzle(int row) { return (row >> 2) & 3; }
@@ -137,7 +157,7 @@ __device__ __forceinline__ void issue_w(const Loader& ld, const Rings<DEPTH>& r,
   const uint32_t kbyte = (uint32_t)j * K_SLOT;
   const int j8 = J8 >= 0 ? J8 : (j & 7);
   // every eighth slot: 16 scale bytes of each routed row (this slot and the next seven)
-  if (j8 == 0) buf16_to_lds(ld.xsc, ld.xscsrc, kbyte >> 5, r.xscale() + ((j >> 3) & 1) * (TILE_X * 16) + wave * 1024);
+  if (j8 == 0) buf16_to_lds_device_scope(ld.xsc, ld.xscsrc, kbyte >> 5, r.xscale() + ((j >> 3) & 1) * (TILE_X * 16) + wave * 1024);
   // every second slot: the tile's weight scales of this pair, one row per thread
   if ((j8 & 1) == 0)
     buf4_to_lds(ld.wsc, ld.wscsrc, (uint32_t)(j >> 1) * ld.wsc_pair_pitch, r.wscale() + (j8 >> 1) * (TILE_W * 4) + wave * 256);
@@ -175,7 +195,7 @@ __device__ __forceinline__ void issue_one(const Loader& ld, const Rings<DEPTH>& 
   constexpr int XL = ODD ? L : L - 2;       // routed-row load 0..3 of this step
   constexpr int WL = ODD ? L - 4 : L - 6;   // weight group
   if constexpr (!ODD && L == 0) {
-    if constexpr (J8 == 0) buf16_to_lds(ld.xsc, ld.xscsrc, kbyte >> 5, r.xscale() + ((j >> 3) & 1) * (TILE_X * 16) + wave * 1024);
+    if constexpr (J8 == 0) buf16_to_lds_device_scope(ld.xsc, ld.xscsrc, kbyte >> 5, r.xscale() + ((j >> 3) & 1) * (TILE_X * 16) + wave * 1024);
   } else if constexpr (!ODD && L == 1) {
     static_assert(ODD || (J8 & 1) == 0, "even steps issue even slots");
     buf4_to_lds(ld.wsc, ld.wscsrc, (uint32_t)(j >> 1) * ld.wsc_pair_pitch, r.wscale() + (J8 >> 1) * (TILE_W * 4) + wave * 256);
@@ -194,8 +214,13 @@ __device__ __forceinline__ void issue_one(const Loader& ld, const Rings<DEPTH>& 
 // (measured on gfx950 with a one-instruction probe).  So a lane reads chunks half and
 // half + 2 of its row; with the XOR swizzle the second is the first with bit 5 flipped.
 __device__ __forceinline__ v8i read_frag(const unsigned char* slot, int off) {
+#ifdef EXP_NOREADS
+  v4i lo = {off, off + 1, off + 2, off + 3}, hi = {off + 4, off + 5, off + 6, off + 7};
+  asm volatile("" : "+v"(lo), "+v"(hi));
+#else
   const v4i lo = *reinterpret_cast<const v4i*>(slot + off);
   const v4i hi = *reinterpret_cast<const v4i*>(slot + (off ^ 32));
+#endif
   v8i r;
   r.s0 = lo.x; r.s1 = lo.y; r.s2 = lo.z; r.s3 = lo.w;
   r.s4 = hi.x; r.s5 = hi.y; r.s6 = hi.z; r.s7 = hi.w;
@@ -281,18 +306,87 @@ __device__ __forceinline__ void mma_step(const Operands& o, const int (&sx)[XFRA
   for (int a = 0; a < WFRAGS; ++a)
 #pragma unroll
     for (int b = 0; b < XFRAGS; ++b)
+#ifndef EXP_NOMFMA
       acc.v[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.w[a], o.x[b], acc.v[a][b], 0, 0, ODD ? 2 : 0,
                                                                     sw[a], ODD ? 2 : 0, sx[b]);
+#else
+      asm volatile("" :: "v"(o.w[a]), "v"(o.x[b]), "v"(sw[a]), "v"(sx[b]));
+#endif
 }
 
-// The gathered part of a tile's loader: routed row -> source row goes through row_token for
-// the gate/up op, a dependent global load.
-__device__ __forceinline__ void gather_rows(const MokGemmResidue& g, const MokGemmTask& t, GemmCarry& c) {
+// Looking ahead.  While a tile is multiplied the framework names the task that comes after it; `stage` asks memory
+// for what that task's prefetch will want first and would otherwise wait for: the row_token entries of its rows
+// (gate/up op) and the readiness counter its rows depend on (down op in a launch of both GEMMs), both straight into
+// LDS.  The loads are younger than everything the running mainloop waits for and have landed when it ends.
+__device__ __forceinline__ bool waits(const MokGemmTask& t, const MokCounters& counters) {
+  return t.wait_target > 0 && t.counter_idx >= 0 && counters.base != nullptr;
+}
+__device__ __forceinline__ void stage(const MokGemmResidue& g, const MokGemmTask& t, const MokCounters& counters) {
+  const int tid = fresh_tid();
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const Rings<2> r;  // the staged areas do not depend on the depth
+  if (t.op == MOK_GEMM_FWD_ROUTED_GATE_UP && g.row_token) {
+    const int row = t.row_begin + tid;
+    const rsrc_t tok = make_rsrc(g.row_token, (uint32_t)g.hidden.rows * 4u);  // one entry per routed row
+    buf4_to_lds(tok, row < t.row_end ? (uint32_t)row * 4u : PAST_THE_END, 0, r.tokens() + wave * 256);
+  }
+  if (waits(t, counters) && wave == 0) {
+    const rsrc_t cnt = make_rsrc(counters.base, (uint32_t)(t.counter_idx + 1) * 4u);
+    buf4_to_lds_device_scope(cnt, (uint32_t)t.counter_idx * 4u, 0, r.peek());  // 64 copies of one word
+    (void)lane;
+  }
+}
+// what `stage` saw of the task's counter: true if the rows the task reads were complete then (or it depends on none)
+__device__ __forceinline__ bool staged_ready(const MokGemmTask& t, const MokCounters& counters) {
+  if (!waits(t, counters)) return true;
+  const Rings<2> r;
+  return *reinterpret_cast<const volatile int32_t*>(r.peek()) >= t.wait_target;
+}
+// Waits until the rows the task reads are complete: one thread polls the counter at device scope, the others wait at
+// the barrier.  A bounded poll: after WAIT_POLLS probes it raises the launch's status word and goes on (the tile then
+// multiplies whatever `hidden` holds), so a launch never spins for ever.
+constexpr uint32_t WAIT_POLLS = 1u << 18;
+__device__ __forceinline__ void wait_rows(const MokGemmTask& t, const MokCounters& counters) {
+  if (!waits(t, counters)) return;
+  if (threadIdx.x == 0) {
+    bool ok = false;
+    for (uint32_t spin = 0; spin < WAIT_POLLS; ++spin) {
+      if (__hip_atomic_load(counters.base + t.counter_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= t.wait_target) {
+        ok = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(8);
+    }
+    if (!ok && counters.status) __hip_atomic_fetch_or(counters.status, (uint32_t)MOK_STATUS_WAIT_GAVE_UP, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+}
+
+// The two operands of a task as this wave sees them, copied out of the residue in one go: a field fetched where it is
+// used is a scalar load and a wait of its own.
+struct Views {
+  MokMxView act;  // routed rows: x (gate/up op) or hidden (down op)
+  MokMxView w;    // weight rows this wave loads: gate or up (by wave) or down
+};
+__device__ __forceinline__ Views views_of(const MokGemmResidue& g, const MokGemmTask& t) {
+  const int wave = __builtin_amdgcn_readfirstlane(fresh_tid() >> 6);
+  const bool gate_up = t.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
+  const MokMxView* a = gate_up ? &g.x : &g.hidden;
+  const MokMxView* w = gate_up ? (wave < WAVES / 2 ? &g.w_gate : &g.w_up) : &g.w_down;
+  return Views{*a, *w};
+}
+
+// The gathered part of a tile's loader: routed row -> source row goes through row_token for the gate/up op, a
+// dependent load: from LDS if the task was staged (tokens of rows past the end are zero there), else from memory.
+__device__ __forceinline__ void gather_rows(const MokGemmResidue& g, const Views& v, const MokGemmTask& t, GemmCarry& c, bool staged) {
   const int tid = fresh_tid();
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const bool gate_up = t.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
-  const MokMxView& act = gate_up ? g.x : g.hidden;
+  const MokMxView& act = v.act;
+  const bool gathered = gate_up && g.row_token;
+  const int32_t* staged_token = reinterpret_cast<const int32_t*>(Rings<2>().tokens());
   const int lrow = lane >> 2;
   const int chunk = 16 * ((lane & 3) ^ swizzle(lrow));
 #pragma unroll
@@ -300,26 +394,30 @@ __device__ __forceinline__ void gather_rows(const MokGemmResidue& g, const MokGe
     const int trow = (wave * X_GROUPS + i) * 16 + lrow;  // tile-local routed row
     const int row = t.row_begin + trow;
     const int safe = row < t.row_end ? row : t.row_end - 1;
-    const int src = (gate_up && g.row_token) ? g.row_token[safe] : safe;
+    const int src = !gathered ? safe : staged ? staged_token[trow] : g.row_token[safe];
     c.xsrc[i] = row < t.row_end ? (uint32_t)src * (uint32_t)act.ld_q + chunk : PAST_THE_END;
   }
   // routed-row scales: thread tid fetches row tid's 16-byte piece
   const int row = t.row_begin + tid;
   const int safe = row < t.row_end ? row : t.row_end - 1;
-  const int src = (gate_up && g.row_token) ? g.row_token[safe] : safe;
+  const int src = !gathered ? safe : staged ? staged_token[tid] : g.row_token[safe];
   c.xscsrc = row < t.row_end ? (uint32_t)src * (uint32_t)act.ld_sc : PAST_THE_END;
 }
 
 // Loader of a tile: lane -> (row lane/4 of a 16-row group, LDS position lane%4); it fetches the
 // chunk that belongs at that position.  Groups start at multiples of 16 rows, so the swizzle
 // of a row only depends on its place in the group.
-__device__ __forceinline__ Loader make_loader(const MokGemmResidue& g, const MokGemmTask& t, const GemmCarry& c) {
+__device__ __forceinline__ Loader make_loader(const Views& v, const MokGemmTask& t, const GemmCarry& c) {
   const int tid = fresh_tid();
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: resources chosen by it stay scalar
   const bool gate_up = t.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
+#ifdef EXP_SAMEW
+  const int expert = 0;
+#else
   const int expert = __builtin_amdgcn_readfirstlane(t.expert);
-  const MokMxView& act = gate_up ? g.x : g.hidden;
+#endif
+  const MokMxView& act = v.act;
   Loader ld;
   const int lrow = lane >> 2;
   const int chunk = 16 * ((lane & 3) ^ swizzle(lrow));
@@ -330,11 +428,15 @@ __device__ __forceinline__ Loader make_loader(const MokGemmResidue& g, const Mok
   ld.xsc = make_rsrc(act.sc, (uint32_t)act.rows * (uint32_t)act.ld_sc);
   ld.dst = wave * X_GROUPS * 1024;
   static_assert(X_GROUPS == W_GROUPS, "one wave offset serves both rings");
-  const MokMxView& wv = gate_up ? (wave < WAVES / 2 ? g.w_gate : g.w_up) : g.w_down;
+  const MokMxView& wv = v.w;
 #pragma unroll
   for (int i = 0; i < W_GROUPS; ++i) {
     const int wl = (wave * W_GROUPS + i) * 16 + lrow;  // tile-local weight row
+#ifdef EXP_SAMEW
+    const int col = (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
+#else
     const int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
+#endif
     ld.wsrc[i] = col < wv.rows ? (uint32_t)col * (uint32_t)K_SLOT + chunk : PAST_THE_END;  // weights are K-tiled: [K/64][rows][64]
   }
   ld.w = make_rsrc(wv.q + (int64_t)expert * wv.expert_pitch_q, (uint32_t)wv.rows * (uint32_t)wv.k);
@@ -400,29 +502,29 @@ __device__ __forceinline__ int loads_younger_than_slot(int slot, int last, int n
 }
 
 template <int DEPTH>
-__device__ __forceinline__ void prefetch(const MokGemmResidue& g, const MokGemmTask& t, GemmCarry& c) {
-  gather_rows(g, t, c);
-  const Loader ld = make_loader(g, t, c);
+__device__ __forceinline__ void prefetch(const MokGemmResidue& g, const MokGemmTask& t, GemmCarry& c, bool staged) {
+  const Views v = views_of(g, t);
+  gather_rows(g, v, t, c, staged);
+  const Loader ld = make_loader(v, t, c);
   const Rings<DEPTH> r;
-  const int n = (t.op == MOK_GEMM_FWD_ROUTED_GATE_UP ? g.x.k : g.hidden.k) / K_SLOT;
+  const int n = v.act.k / K_SLOT;
   issue_step(ld, r, -DEPTH, n, 0, 1, 0);
   issue_step(ld, r, 1 - DEPTH, n, 0, 1, 1);
 }
 
 template <int DEPTH>
 __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmTask& t, AccFrag& acc,
-                                         const GemmCarry& carry) {
+                                         const GemmCarry& carry, const MokGemmTask* upcoming, const MokCounters& counters) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31;
   const int half = lane >> 5;
-  const bool gate_up = t.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
-  const MokMxView& act = gate_up ? g.x : g.hidden;
-  const int n = act.k / K_SLOT;  // the host rejects a contraction length that is not a multiple of 64
+  const Views v = views_of(g, t);
+  const int n = v.act.k / K_SLOT;  // the host rejects a contraction length that is not a multiple of 64
   constexpr int XDEPTH = DEPTH + 1;
   const Rings<DEPTH> r;
-  const Loader ld = make_loader(g, t, carry);
+  const Loader ld = make_loader(v, t, carry);
 
   // ---- per-fragment LDS read offsets (first block) ------------------------------------
   int xoff[XFRAGS], woff[WFRAGS], xscoff[XFRAGS], wscoff[WFRAGS];
@@ -456,13 +558,19 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   // ---- rest of the prologue (steps -DEPTH and 1-DEPTH were issued by `prefetch`), then slot 0's operands
 #pragma unroll
   for (int u = 2 - DEPTH; u < 0; ++u) issue_step(ld, r, u, n, (u + DEPTH) & ~1, ((u + DEPTH) & ~1) + 1, u + DEPTH);
+  // The look-ahead loads go here, behind the prologue's: the waits below count the loads that may still be in flight
+  // behind the slot they need, and loads return in order, so one or two more of the youngest only make the next few
+  // waits ask for as many more of the oldest.
+#ifndef EXP_NO_STAGE
+  if (upcoming->op != 0) stage(g, *upcoming, counters);
+#endif
   wait_loads_and_reads_dyn(loads_younger_than_slot<DEPTH>(0, -1, n));
   wg_barrier();
   auto xnext = [](int b, int by) {  // (b + by) mod XDEPTH for 0 <= b < XDEPTH, 0 <= by <= XDEPTH
     const int c = b + by;
     return c >= XDEPTH ? c - XDEPTH : c;
   };
-  if (wave_idle(t, (gate_up ? g.w_gate : g.w_down).rows)) {
+  if (wave_idle(t, v.w.rows)) {
     // Loader only.  Same loop bounds as the multiplying waves below, one wait + barrier + issue
     // per step, so every wave of the workgroup passes the same number of barriers.
     int xb = 0, wb = 0;
@@ -528,8 +636,12 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       auto place = [&](auto I_) {
         constexpr int I = decltype(I_)::value;
         constexpr int A = I / XFRAGS, B = I % XFRAGS;
+#ifndef EXP_NOMFMA
         acc.v[A][B] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cur.w[A], cur.x[B], acc.v[A][B], 0, 0, ODD ? 2 : 0,
                                                                       sw[A], ODD ? 2 : 0, sx[B]);
+#else
+        asm volatile("" :: "v"(cur.w[A]), "v"(cur.x[B]), "v"(sw[A]), "v"(sx[B]));
+#endif
         __builtin_amdgcn_sched_barrier(0);  // the MFMA goes first: the pipe is what must not wait
         if constexpr (I == 1) {
           wait_loads_and_reads<ODD ? STEADY_ODD : STEADY_EVEN>();
@@ -700,34 +812,64 @@ __device__ __forceinline__ void store_down(const MokGemmResidue& g, const MokGem
 }  // namespace mok_gemm_owner
 
 extern "C" __device__ void mok_gemm_init(const void* view) { (void)view; }
+// Nothing to give back: the owner holds no barriers or tensor memory of its own (campaigns/mok/port/gemm/gemm_abi.h:52-54
+// exports init, fini and fwd; init and fini are where the reference sets up and frees its mbarriers and TMEM columns).
+extern "C" __device__ void mok_gemm_fini(const void* view) { (void)view; }
 
 static __device__ __forceinline__ const MokGemmResidue& mok_gemm_residue(const void* view) {
   return *static_cast<const MokGemmResidue*>(static_cast<const pipelink_host_view*>(view)->residue);
 }
 
-// Starts the loads of a tile's first two slots and leaves the gathered row offsets in *carry.
+// Looks ahead to a task outside a mainloop (a workgroup's first tile): asks for the task's row tokens and readiness
+// counter.  The caller waits for its loads and passes a workgroup barrier before it calls mok_gemm_ready / _prefetch.
+extern "C" __device__ void mok_gemm_stage(const void* view, const MokGemmTask* task, const MokCounters* counters) {
+  mok_gemm_owner::stage(mok_gemm_residue(view), *task, *counters);
+}
+
+// True if the rows the staged task reads were complete when it was staged (always, for a task that depends on none).
+extern "C" __device__ bool mok_gemm_ready(const void* view, const MokGemmTask* task, const MokCounters* counters) {
+  (void)view;
+  return mok_gemm_owner::staged_ready(*task, *counters);
+}
+
+// Waits (bounded) until the rows the task reads are complete; raises MOK_STATUS_WAIT_GAVE_UP in *counters->status
+// if they are not after 2^18 polls.  Must not be called while the workgroup holds a tile whose results others wait for.
+extern "C" __device__ void mok_gemm_wait(const void* view, const MokGemmTask* task, const MokCounters* counters) {
+  (void)view;
+  mok_gemm_owner::wait_rows(*task, *counters);
+}
+
+// Starts the loads of a tile's first two slots and leaves the gathered row offsets in *carry.  The task must have been
+// staged, and the rows it reads must be complete (mok_gemm_ready / mok_gemm_wait).
 // Only touches the head buffers: the caller may run it between the previous tile's mainloop
 // and that tile's epilogue.
 extern "C" __device__ void mok_gemm_prefetch(const void* view, const MokGemmTask* task, mok::GemmCarry* carry) {
   const auto& g = mok_gemm_residue(view);
   switch (pipelink_mok_gemm_depth()) {  // a link-time constant: one case survives
-    case 2: mok_gemm_owner::prefetch<2>(g, *task, *carry); break;
-    default: mok_gemm_owner::prefetch<4>(g, *task, *carry); break;
+#ifdef EXP_NO_STAGE
+    case 2: mok_gemm_owner::prefetch<2>(g, *task, *carry, false); break;
+    default: mok_gemm_owner::prefetch<4>(g, *task, *carry, false); break;
+#else
+    case 2: mok_gemm_owner::prefetch<2>(g, *task, *carry, true); break;
+    default: mok_gemm_owner::prefetch<4>(g, *task, *carry, true); break;
+#endif
   }
 }
 
 // Runs the mainloop of one tile whose prefetch has been issued (same task, same carry) and
 // leaves the fp32 accumulator in *acc: for the activation owner (gate/up op) or for
-// mok_gemm_store (down op).
+// mok_gemm_store (down op).  `upcoming`, unless its op is 0, is the task this workgroup runs next: it is staged
+// (see mok_gemm_stage) behind the tile's first loads, and is ready for mok_gemm_ready / _prefetch when the call returns.
+// *phase counts the tiles this workgroup has multiplied.
 extern "C" __device__ void mok_gemm_fwd(const void* view, const MokGemmTask* task, const MokCounters* counters,
-                                        uint32_t* phase, mok::AccFrag* acc, const mok::GemmCarry* carry) {
-  (void)counters;
-  (void)phase;
+                                        uint32_t* phase, mok::AccFrag* acc, const mok::GemmCarry* carry,
+                                        const MokGemmTask* upcoming) {
   const auto& g = mok_gemm_residue(view);
   switch (pipelink_mok_gemm_depth()) {
-    case 2: mok_gemm_owner::mainloop<2>(g, *task, *acc, *carry); break;
-    default: mok_gemm_owner::mainloop<4>(g, *task, *acc, *carry); break;
+    case 2: mok_gemm_owner::mainloop<2>(g, *task, *acc, *carry, upcoming, *counters); break;
+    default: mok_gemm_owner::mainloop<4>(g, *task, *acc, *carry, upcoming, *counters); break;
   }
+  ++*phase;
 }
 
 // Down op only: rounds the accumulator to bf16 and stores the tile of y.
@@ -747,20 +889,33 @@ PL_PARAMS(MokGemmResidue);
 PL_TOPOLOGY(true, "static");
 PL_VARIANT(0, {{"pipelink_mok_precision", 1}});  // MXFP8 (campaigns/mok/port/include/mok_abi.h: MOK_PRECISION_MXFP8)
 PL_EXPORT(mok_gemm_init, mok_gemm_init, "extern \"C\" __device__ void mok_gemm_init(const void* view);");
+PL_EXPORT(mok_gemm_fini, mok_gemm_fini, "extern \"C\" __device__ void mok_gemm_fini(const void* view);");
+PL_EXPORT(mok_gemm_stage, mok_gemm_stage,
+          "extern \"C\" __device__ void mok_gemm_stage(const void* view, const MokGemmTask* task, const MokCounters* counters);");
+PL_EXPORT(mok_gemm_ready, mok_gemm_ready,
+          "extern \"C\" __device__ bool mok_gemm_ready(const void* view, const MokGemmTask* task, const MokCounters* counters);");
+PL_EXPORT(mok_gemm_wait, mok_gemm_wait,
+          "extern \"C\" __device__ void mok_gemm_wait(const void* view, const MokGemmTask* task, const MokCounters* counters);");
 PL_EXPORT(mok_gemm_prefetch, mok_gemm_prefetch,
           "extern \"C\" __device__ void mok_gemm_prefetch(const void* view, const MokGemmTask* task, mok::GemmCarry* carry);");
 PL_EXPORT(mok_gemm_fwd, mok_gemm_fwd,
           "extern \"C\" __device__ void mok_gemm_fwd(const void* view, const MokGemmTask* task, "
-          "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc, const mok::GemmCarry* carry);");
+          "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc, const mok::GemmCarry* carry, "
+          "const MokGemmTask* upcoming);");
 PL_EXPORT(mok_gemm_store, mok_gemm_store,
           "extern \"C\" __device__ void mok_gemm_store(const void* view, const MokGemmTask* task, const mok::AccFrag* acc);");
 PL_SERVE(gemm_init, "mok_gemm_init");
+PL_SERVE(gemm_fini, "mok_gemm_fini");
+PL_SERVE(gemm_stage, "mok_gemm_stage");
+PL_SERVE(gemm_ready, "mok_gemm_ready");
+PL_SERVE(gemm_wait, "mok_gemm_wait");
 PL_SERVE(gemm_prefetch, "mok_gemm_prefetch");
 PL_SERVE(gemm_fwd, "mok_gemm_fwd");
 PL_SERVE(gemm_store, "mok_gemm_store");
 // head, live for the whole kernel: the first two 16 KB buffers of the routed-row ring and of the weight
-// ring, four 1 KB buffers of weight scales, two 4 KB buffers of routed-row scales
-PL_CLAIM("pipelink_mok_gemm_head", "smem", 4 * 16384 + 4096 + 8192, 1024, "kernel");
+// ring, four 1 KB buffers of weight scales, two 4 KB buffers of routed-row scales, the staged task's row tokens (1 KB)
+// and readiness counter (256 B)
+PL_CLAIM("pipelink_mok_gemm_head", "smem", 4 * 16384 + 4096 + 8192 + 1024 + 256, 1024, "kernel");
 // arena, live during the GEMM phase: the other buffers of the two rings -- depth + 1 - 2 routed-row
 // buffers and depth - 2 weight buffers, (2 * depth - 3) x 16 KB
 PL_CLAIM_RING("pipelink_mok_gemm_arena", "smem", -3 * 16384, "pipelink_mok_gemm_depth", 32768, 1024, "phase:instr_gemm");

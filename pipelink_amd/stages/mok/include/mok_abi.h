@@ -16,12 +16,17 @@
 #ifndef MOKCOUNTERS_DEFINED
 #define MOKCOUNTERS_DEFINED
 typedef struct MokCounters {
-  int32_t* base; /* counter workspace lent by the framework to every op call */
+  int32_t* base; /* dependency counters lent by the framework to every op call: base[t] counts the gate/up tiles of
+                    routed-row tile t whose `hidden` columns are in memory (campaigns/mok/port/gemm/gemm.cu:364-382:
+                    the reference's readiness counts); null when the launch runs one GEMM only */
+  uint32_t* status; /* sticky word of the launch: MOK_STATUS_* bits, raised by a wait that gave up */
 } MokCounters;
 #endif
+enum { MOK_STATUS_WAIT_GAVE_UP = 1 };
 
 /* op codes keep the reference's names; GATE and UP of one tile are issued as one task */
 enum {
+  MOK_FWD_BOTH = 0,                /* framework params only: gate/up tiles, then down tiles, in one launch */
   MOK_GEMM_FWD_ROUTED_GATE_UP = 3, /* = MOK_GEMM_FWD_ROUTED_GATE of the reference */
   MOK_GEMM_FWD_ROUTED_DOWN = 5
 };
@@ -36,6 +41,9 @@ typedef struct MokGemmTask {
   int32_t row_end;   /* one past the expert's last routed row; rows >= row_end are padding */
   int32_t col_begin; /* first output column of the tile (per weight matrix) */
   int32_t task_idx;  /* running index of the tile in the schedule */
+  int32_t counter_idx; /* readiness counter of the tile's routed-row tile (a launch of both GEMMs), or -1 */
+  int32_t wait_target; /* down op: value that counter must have reached before the tile's rows of `hidden` are read
+                          (the number of gate/up column tiles); 0 = the tile waits for nothing */
   uint32_t flags;
 } MokGemmTask;
 #endif
@@ -46,6 +54,7 @@ typedef struct MokActTask {
   int32_t op;        /* MOK_ACT_FWD_ROUTED */
   int32_t row_begin, row_end, col_begin;
   int32_t task_idx;
+  int32_t counter_idx; /* counter to bump once the tile's `hidden` columns are in memory, or -1 */
   uint32_t flags;
 } MokActTask;
 #endif
@@ -92,13 +101,19 @@ typedef struct MokActResidue {
 /* Params of the framework role: the schedule. */
 typedef struct MokFrameworkParams {
   const int32_t* tokens_per_expert; /* [E] */
-  int32_t* expert_row_begin;        /* [E+1] exclusive prefix sum of tokens_per_expert (workspace) */
-  int32_t* expert_tile_begin;       /* [E+1] exclusive prefix sum of row tiles (workspace) */
+  uint32_t* workspace;              /* MOK_WS_* words + one counter per routed-row tile; all zero before a launch,
+                                       and the launch leaves them zero (except the status word) */
   int32_t num_experts;
-  int32_t op;                       /* which GEMM this launch runs */
-  int32_t num_col_tiles;
-  int32_t reserved;
+  int32_t op;                       /* which GEMM this launch runs, or MOK_FWD_BOTH */
+  int32_t num_col_tiles_gate_up;    /* column tiles of the gate/up GEMM (128 gate + 128 up columns each) */
+  int32_t num_col_tiles_down;       /* column tiles of the down GEMM (256 columns each) */
 } MokFrameworkParams;
+/* workspace words */
+enum {
+  MOK_WS_STATUS = 0,    /* sticky MOK_STATUS_* bits; the host reads and clears it */
+  MOK_WS_FINISHED = 1,  /* workgroups that have left the launch; the last one clears the counters */
+  MOK_WS_COUNTERS = 32  /* first readiness counter */
+};
 
 /* The shared scalars every owner of this pipeline is handed (ids of include/plk_host_abi_v2.h); a stage source
  * invokes this among its annotations, after <pipelink/stage.hpp>. */
@@ -114,7 +129,8 @@ typedef struct MokFrameworkParams {
   PL_HOST_SCALAR(61, "mok.ld_q_h", "i64");                \
   PL_HOST_SCALAR(62, "mok.ld_q_i", "i64");                \
   PL_HOST_SCALAR(63, "mok.ld_sc_h", "i64");               \
-  PL_HOST_SCALAR(64, "mok.ld_sc_i", "i64")
+  PL_HOST_SCALAR(64, "mok.ld_sc_i", "i64");               \
+  PL_HOST_SCALAR(65, "mok.workspace_words", "i64")
 
 /* First argument of every owner export (pack/include/pipelink/host_view.h in the reference). */
 #ifndef PIPELINK_HOST_VIEW_DEFINED

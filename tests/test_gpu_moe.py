@@ -51,7 +51,7 @@ def _run(sess, inp, H, I, pitch_h=None, pitch_i=None, limit=7.0):
     y = torch.full((rows, H), float("nan"), dtype=torch.bfloat16, device=dev)
     prob = sess.problem(hidden_q=hq, hidden_sc=hsc, y=y, swiglu_limit=limit, **d)
     sess.forward(prob)
-    torch.cuda.synchronize()
+    assert sess.status() == 0   # waits for the stream; a bounded dependency wait that gave up would show here
     return hq[:, :I].cpu().numpy(), hsc.cpu().numpy(), y.cpu()
 
 
@@ -90,6 +90,11 @@ def test_forward_matches_oracle(cell, T, H, I, E, k, seed, conc):
     assert moe_ffn.rel_frobenius(hid, hid_ref) <= TOL
     nb = I // 32
     assert (hsc[:, :nb] != ref["hidden_sc"][:, :nb]).mean() < 1e-3   # block scales agree except at exact ties
+    # rows of hidden_q padded to whole cache lines: the forward is then ONE launch whose down tiles wait on readiness
+    # counters, and must write the bytes the two launches wrote
+    hq1, hsc1, y1 = _run(cell[0], inp, H, I, pitch_i=(I + 127) // 128 * 128)
+    assert np.array_equal(hq1, hq) and np.array_equal(hsc1[:, :nb], hsc[:, :nb])
+    assert torch.equal(y1.view(torch.int16), y.view(torch.int16))
 
 
 def _random_cases(n, seed):
@@ -111,6 +116,60 @@ def _random_cases(n, seed):
 @pytest.mark.parametrize("T,H,I,E,k,seed,conc", _random_cases(16, 7))
 def test_forward_matches_oracle_on_seeded_random_shapes(cell, T, H, I, E, k, seed, conc):
     test_forward_matches_oracle(cell, T, H, I, E, k, seed, conc)
+
+
+def test_tiles_at_the_end_of_an_experts_rows(cell):
+    """Experts of 257, 1025 and 1080 rows: a second / fifth row tile that holds 1, 1 and 56 rows, next to full tiles of
+    the same expert; one expert of exactly 256 rows and an empty one."""
+    from pipelink_amd.host import mok_inputs
+
+    T, H, I = 512, 256, 384
+    inp = mok_inputs.generate(T, H, I, 5, 1, seed=31, counts=[257, 1025, 0, 1080, 256])
+    for pitch in (None, 384):   # two launches; one launch
+        hq, hsc, y = _run(cell[0], inp, H, I, pitch_i=pitch)
+        ref = _oracle(inp)
+        yy = y.float().numpy()
+        assert not np.isnan(yy).any()
+        assert moe_ffn.rel_frobenius(yy, ref["y"]) <= TOL
+        assert moe_ffn.rel_frobenius(mxfp8.mx_dequantize(hq, hsc), mxfp8.mx_dequantize(ref["hidden_q"], ref["hidden_sc"])) <= TOL
+
+
+def test_one_launch_forward_twice_on_the_same_buffers(cell):
+    """Two forwards in a row that share hidden / y buffers but not inputs: the second must not read anything of the
+    first (its `hidden` rows as an XCD's cache may still hold them) -- against a forward into fresh buffers; and a
+    one-launch forward equals its two passes launched one after the other."""
+    from pipelink_amd.host import mok_inputs
+    from pipelink_amd.host.mok import scale_pitch, weight_codes_to_k64_tiled, weight_scales_to_slot_major
+
+    T, H, I, E, k, PITCH = 2048, 512, 640, 8, 2, 640
+    dev = torch.device("cuda:0")
+    sess = cell[0]
+    rows = T * k
+    hq = torch.empty((rows, PITCH), dtype=torch.uint8, device=dev)
+    hsc = torch.empty((rows, scale_pitch(I)), dtype=torch.uint8, device=dev)
+    y = torch.empty((rows, H), dtype=torch.bfloat16, device=dev)
+    got, keep = [], []
+    for seed in (41, 42):
+        inp = mok_inputs.generate(T, H, I, E, k, seed=seed)
+        d = {n: v.to(dev) for n, v in inp.__dict__.items()}
+        d["w_gate_sc"], d["w_up_sc"] = weight_scales_to_slot_major(d["w_gate_sc"], H), weight_scales_to_slot_major(d["w_up_sc"], H)
+        d["w_down_sc"] = weight_scales_to_slot_major(d["w_down_sc"], I)
+        d["w_gate_q"], d["w_up_q"] = weight_codes_to_k64_tiled(d["w_gate_q"], H), weight_codes_to_k64_tiled(d["w_up_q"], H)
+        d["w_down_q"] = weight_codes_to_k64_tiled(d["w_down_q"], I)
+        keep.append(d)
+        prob = sess.problem(hidden_q=hq, hidden_sc=hsc, y=y, **d)
+        sess.forward(prob)                       # no poison, no wait in between: back to back on one stream
+        if seed == 42:
+            assert sess.status() == 0
+            got = [hq[:, :I].cpu().numpy(), hsc.cpu().numpy(), y.cpu()]
+            hq.fill_(0xFF); hsc.fill_(0xFF); y.fill_(float("nan"))
+            sess.forward(prob, which=1)
+            sess.forward(prob, which=2)
+            torch.cuda.synchronize()
+            assert np.array_equal(hq[:, :I].cpu().numpy(), got[0]) and torch.equal(y.cpu().view(torch.int16), got[2].view(torch.int16))
+            fresh = _run(sess, inp, H, I, pitch_i=PITCH)
+            assert np.array_equal(fresh[0], got[0]) and np.array_equal(fresh[1][:, :I // 32], got[1][:, :I // 32])
+            assert torch.equal(fresh[2].view(torch.int16), got[2].view(torch.int16))
 
 
 def test_linked_and_one_unit_images_are_byte_identical(cell):
@@ -211,8 +270,9 @@ def test_broker_route_gives_the_same_bytes_as_the_forward_entry(cell):
     from pipelink_amd.stages.mok import build as mok_build
 
     T, H, I, E, k = 300, 320, 192, 4, 2
+    PITCH = 256   # rows of hidden_q that are whole cache lines: both GEMMs may run in one launch
     inp = mok_inputs.generate(T, H, I, E, k, seed=1)
-    want = _run(cell[0], inp, H, I)
+    want = _run(cell[0], inp, H, I, pitch_i=PITCH)
     dev = torch.device("cuda:0")
     d = {n: v.to(dev) for n, v in inp.__dict__.items()}
     t = dict(x_q=d["x_q"], x_sc=d["x_sc"], row_token=d["row_token"], tokens_per_expert=d["tokens_per_expert"],
@@ -220,26 +280,33 @@ def test_broker_route_gives_the_same_bytes_as_the_forward_entry(cell):
              w_up_q=weight_codes_to_k64_tiled(d["w_up_q"], H), w_up_sc=weight_scales_to_slot_major(d["w_up_sc"], H),
              w_down_q=weight_codes_to_k64_tiled(d["w_down_q"], I), w_down_sc=weight_scales_to_slot_major(d["w_down_sc"], I))
     rows = int(inp.tokens_per_expert.sum())
-    t["hidden_q"] = torch.full((rows, I), 0xFF, dtype=torch.uint8, device=dev)
-    t["hidden_sc"] = torch.full((rows, scale_pitch(I)), 0xFF, dtype=torch.uint8, device=dev)
-    t["y"] = torch.full((rows, H), float("nan"), dtype=torch.bfloat16, device=dev)
+    words = 32 + (rows + 255) // 256 + E
+    t["hidden_q"] = torch.empty((rows, PITCH), dtype=torch.uint8, device=dev)
+    t["hidden_sc"] = torch.empty((rows, scale_pitch(I)), dtype=torch.uint8, device=dev)
+    t["y"] = torch.empty((rows, H), dtype=torch.bfloat16, device=dev)
+    t["workspace"] = torch.zeros(words, dtype=torch.int32, device=dev)
     res = lambda n: broker.Resource(t[n].data_ptr(), t[n].numel() * t[n].element_size())
-    resources = {"mok.framework": {"tokens_per_expert": res("tokens_per_expert")},
+    resources = {"mok.framework": {"tokens_per_expert": res("tokens_per_expert"), "workspace": res("workspace")},
                  "mok.gemm": {n: res(n) for n in ("x_q", "x_sc", "w_gate_q", "w_gate_sc", "w_up_q", "w_up_sc", "w_down_q",
                                                   "w_down_sc", "hidden_q", "hidden_sc", "y", "row_token")},
                  "mok.act": {"hidden_q": res("hidden_q"), "hidden_sc": res("hidden_sc")}}
     scalars = {"mok.num_local_tokens": T, "mok.hidden": H, "mok.intermediate": I, "mok.num_local_experts": E,
                "mok.swiglu_limit": 7.0, "mok.pass": 1, "mok.precision": 1, "mok.routed_rows": rows, "mok.ld_q_h": H,
-               "mok.ld_q_i": I, "mok.ld_sc_h": scale_pitch(H), "mok.ld_sc_i": scale_pitch(I)}
+               "mok.ld_q_i": PITCH, "mok.ld_sc_h": scale_pitch(H), "mok.ld_sc_i": scale_pitch(I), "mok.workspace_words": words}
     paths = mok_build.images()
     link = json.loads(paths["link_json"].read_text())
     be = HipBackend(0, torch.cuda.current_stream().cuda_stream)
-    for pass_ in (1, 2):
-        with broker.open_host(link, paths["linked"].read_bytes(), resources, dict(scalars, **{"mok.pass": pass_}), be) as s:
-            s.launch()
-            be.synchronize()
-    assert np.array_equal(t["hidden_q"].cpu().numpy(), want[0]) and np.array_equal(t["hidden_sc"].cpu().numpy(), want[1])
-    assert torch.equal(t["y"].cpu().view(torch.int16), want[2].view(torch.int16))
+    for passes in ((1, 2), (0,)):   # two launches, then both GEMMs in one
+        t["hidden_q"].fill_(0xFF)
+        t["hidden_sc"].fill_(0xFF)
+        t["y"].fill_(float("nan"))
+        for pass_ in passes:
+            with broker.open_host(link, paths["linked"].read_bytes(), resources, dict(scalars, **{"mok.pass": pass_}), be) as s:
+                s.launch()
+                be.synchronize()
+        assert np.array_equal(t["hidden_q"][:, :I].cpu().numpy(), want[0]) and np.array_equal(t["hidden_sc"].cpu().numpy(), want[1])
+        assert torch.equal(t["y"].cpu().view(torch.int16), want[2].view(torch.int16))
+        assert not t["workspace"].cpu().any()   # the launch left its counters at zero and raised no status bit
 
 
 def test_launch_verb_runs_both_passes_through_the_providers(cell, tmp_path):
@@ -267,10 +334,12 @@ def test_launch_verb_runs_both_passes_through_the_providers(cell, tmp_path):
         data = tensor.cpu().contiguous().numpy().tobytes()
         (tmp_path / f"{name}.bin").write_bytes(data)
         resources[name] = {"data": f"{name}.bin", "allocation_bytes": len(data)}
+    words = 32 + (rows + 255) // 256 + E
+    resources["workspace"] = {"data": None, "allocation_bytes": 4 * words}   # zeroed by the fixture
     sizes = {"hidden_q": rows * I, "hidden_sc": rows * scale_pitch(I), "y": rows * H * 2}
     scalars = {"mok.num_local_tokens": T, "mok.hidden": H, "mok.intermediate": I, "mok.num_local_experts": E,
                "mok.swiglu_limit": 7.0, "mok.pass": 1, "mok.precision": 1, "mok.routed_rows": rows, "mok.ld_q_h": H,
-               "mok.ld_q_i": I, "mok.ld_sc_h": scale_pitch(H), "mok.ld_sc_i": scale_pitch(I)}
+               "mok.ld_q_i": I, "mok.ld_sc_h": scale_pitch(H), "mok.ld_sc_i": scale_pitch(I), "mok.workspace_words": words}
     link = str(mok_build.images()["link_json"])
     providers = [arg for g in ("mok.framework.params", "mok.gemm.params", "mok.act.params") for arg in ("--provider", f"{g}={LIB_PATH}")]
     first = dict(resources, hidden_q={"data": None, "allocation_bytes": sizes["hidden_q"], "output": "hidden_q.bin"},
@@ -399,11 +468,12 @@ def test_benchmark_configuration_properties(cell):
     assert np.array_equal(hq2, hq[perm]) and np.array_equal(hsc2[:, :I // 32], hsc[perm][:, :I // 32])
     _, _, y3 = _run(cell[1], host, H, I)
     assert np.array_equal(y3.view(torch.int16).numpy(), yb)                        # (3)
-    e = int(np.argmin(counts))                                                      # (4) the smallest expert
-    lo, n = int(offsets[e]), int(counts[e])
-    one = np.zeros_like(counts)
-    one[e] = n
-    ref = moe_ffn.moe_ffn_forward(host.x_q.numpy(), host.x_sc.numpy(), host.w_gate_q.numpy(), host.w_gate_sc.numpy(),
-                                  host.w_up_q.numpy(), host.w_up_sc.numpy(), host.w_down_q.numpy(), host.w_down_sc.numpy(),
-                                  one, host.row_token.numpy()[lo:lo + n])
-    assert moe_ffn.rel_frobenius(y.float().numpy()[lo:lo + n], ref["y"]) <= TOL
+    # (4) the smallest expert, and the largest: 1080 rows, a fifth row tile with 56 rows in it
+    for e in (int(np.argmin(counts)), int(np.argmax(counts))):
+        lo, n = int(offsets[e]), int(counts[e])
+        one = np.zeros_like(counts)
+        one[e] = n
+        ref = moe_ffn.moe_ffn_forward(host.x_q.numpy(), host.x_sc.numpy(), host.w_gate_q.numpy(), host.w_gate_sc.numpy(),
+                                      host.w_up_q.numpy(), host.w_up_sc.numpy(), host.w_down_q.numpy(), host.w_down_sc.numpy(),
+                                      one, host.row_token.numpy()[lo:lo + n])
+        assert moe_ffn.rel_frobenius(y.float().numpy()[lo:lo + n], ref["y"]) <= TOL

@@ -18,13 +18,18 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 SCALARS = {"mok.num_local_tokens": 512, "mok.hidden": 320, "mok.intermediate": 192, "mok.num_local_experts": 4,
            "mok.swiglu_limit": 7.0, "mok.pass": 1, "mok.precision": 1, "mok.routed_rows": 1024, "mok.ld_q_h": 384,
-           "mok.ld_q_i": 256, "mok.ld_sc_h": 16, "mok.ld_sc_i": 16}
+           "mok.ld_q_i": 256, "mok.ld_sc_h": 16, "mok.ld_sc_i": 16,
+           "mok.workspace_words": 32 + 1024 // 256 + 4}   # status and counter words + one counter per possible row tile
 # the owner inventory is what the built pipeline's link recorded from the stages' PL_HOST_* declarations
-HOST = json.loads(open(os.path.join(ROOT, "pipelink_amd", "stages", "mok", "build", "link", "link.json")).read())["host"]
-LINK = {"threads": 256, "dyn_smem_bytes": 161800, "kernel_symbol": "pipelink_kernel", "workgroups_per_cu": 1, "host": HOST,
-        "params": {"total_bytes": 344, "entries": [{"stage_id": "mok.framework", "offset": 0, "bytes": 40},
-                                                   {"stage_id": "mok.gemm", "offset": 40, "bytes": 264},
-                                                   {"stage_id": "mok.act", "offset": 304, "bytes": 40}]}}
+_LINK_JSON = os.path.join(ROOT, "pipelink_amd", "stages", "mok", "build", "link", "link.json")
+if not os.path.exists(_LINK_JSON):
+    pytest.skip("the routed-expert FFN cell is not built (run __graft_entry__.build()): " + _LINK_JSON, allow_module_level=True)
+_BUILT = json.loads(open(_LINK_JSON).read())
+HOST = _BUILT["host"]
+LINK = {"threads": 256, "dyn_smem_bytes": _BUILT["dyn_smem_bytes"], "kernel_symbol": "pipelink_kernel", "workgroups_per_cu": 1,
+        "host": HOST, "params": _BUILT["params"]}
+_AT = {e["stage_id"]: (e["offset"], e["offset"] + e["bytes"]) for e in LINK["params"]["entries"]}
+FW, GEMM, ACT = _AT["mok.framework"], _AT["mok.gemm"], _AT["mok.act"]
 GROUPS = {g["owner"]: g for g in HOST["groups"]}
 
 
@@ -50,7 +55,8 @@ def test_abi_report_matches_the_ctypes_mirrors():
     for stage, group in GROUPS.items():
         rep = broker.Owner(lib, group).report()          # raises on any size / alignment / digest mismatch
         assert rep.entry_count == 20 + len(group["provider"]["abi_types"])
-    assert sizeof(broker.MokGemmResidue) == 264 and sizeof(broker.MokActResidue) == 40 and sizeof(broker.MokFrameworkParams) == 40
+    assert sizeof(broker.MokGemmResidue) == 264 and sizeof(broker.MokActResidue) == 40 and sizeof(broker.MokFrameworkParams) == 32
+    assert (FW, GEMM, ACT) == ((0, 32), (32, 296), (296, 336))
 
 
 def test_abi_report_rejects_wrong_version_capacity_and_ids():
@@ -72,13 +78,15 @@ def test_abi_report_rejects_wrong_version_capacity_and_ids():
 def test_plan_builds_the_same_image_as_the_structs_say():
     res = _resources()
     image, geometry, owners = broker.plan(LINK, res, SCALARS, compute_units=256)
-    assert len(image) == 344 and geometry["block"] == (256, 1, 1) and geometry["dyn_lds"] == 161800
+    assert len(image) == 336 and geometry["block"] == (256, 1, 1) and geometry["dyn_lds"] == LINK["dyn_smem_bytes"]
     assert geometry["grid"][0] % 8 == 0 and 0 < geometry["grid"][0] <= 256
-    fw = broker.MokFrameworkParams.from_buffer_copy(image[0:40])
-    g = broker.MokGemmResidue.from_buffer_copy(image[40:304])
-    a = broker.MokActResidue.from_buffer_copy(image[304:344])
+    fw = broker.MokFrameworkParams.from_buffer_copy(image[FW[0]:FW[1]])
+    g = broker.MokGemmResidue.from_buffer_copy(image[GEMM[0]:GEMM[1]])
+    a = broker.MokActResidue.from_buffer_copy(image[ACT[0]:ACT[1]])
     assert fw.tokens_per_expert == res["mok.framework"]["tokens_per_expert"].address
-    assert (fw.num_experts, fw.op, fw.num_col_tiles) == (4, 3, 2)             # gate/up: ceil(192 / 128) column tiles
+    assert fw.workspace == res["mok.framework"]["workspace"].address
+    # gate/up: ceil(192 / 128) column tiles, down: ceil(320 / 256)
+    assert (fw.num_experts, fw.op, fw.num_col_tiles_gate_up, fw.num_col_tiles_down) == (4, 3, 2, 2)
     assert (g.x.q, g.x.rows, g.x.k, g.x.ld_q, g.x.ld_sc) == (res["mok.gemm"]["x_q"].address, 512, 320, 384, 16)
     assert (g.w_gate.rows, g.w_gate.k, g.w_gate.ld_q, g.w_gate.expert_pitch_q, g.w_gate.expert_pitch_sc) == \
         (192, 320, 64, 192 * 320, 3 * 192 * 4)
@@ -90,14 +98,21 @@ def test_plan_builds_the_same_image_as_the_structs_say():
         assert o.release(o.session) == 0                  # null sessions release fine
     down = dict(SCALARS, **{"mok.pass": 2})
     image2, _, _ = broker.plan(LINK, res, down, compute_units=256)
-    fw2 = broker.MokFrameworkParams.from_buffer_copy(image2[0:40])
-    assert (fw2.op, fw2.num_col_tiles) == (5, 2) and image2[40:] == image[40:]
+    fw2 = broker.MokFrameworkParams.from_buffer_copy(image2[FW[0]:FW[1]])
+    assert fw2.op == 5 and image2[FW[1]:] == image[FW[1]:]
+    # both GEMMs in one launch: op 0, and only with rows of `hidden` that are whole cache lines
+    both, _, _ = broker.plan(LINK, res, dict(SCALARS, **{"mok.pass": 0}), compute_units=256)
+    assert broker.MokFrameworkParams.from_buffer_copy(both[FW[0]:FW[1]]).op == 0 and both[FW[1]:] == image[FW[1]:]
+    with pytest.raises(PlkError) as err:
+        odd = dict(SCALARS, **{"mok.pass": 0, "mok.ld_q_i": 192})
+        broker.plan(LINK, _resources(odd), odd, compute_units=256)
+    assert err.value.status == 3
 
 
 def test_optional_row_token_channel_may_be_absent():
     res = _resources(row_token=False)
     image, _, _ = broker.plan(LINK, res, SCALARS, compute_units=256)
-    assert broker.MokGemmResidue.from_buffer_copy(image[40:304]).row_token is None
+    assert broker.MokGemmResidue.from_buffer_copy(image[GEMM[0]:GEMM[1]]).row_token is None
 
 
 @pytest.mark.parametrize("mutate,status", [
@@ -150,7 +165,8 @@ def test_owner_inventory_comes_from_the_link():
                                                      "w_down_sc", "hidden_q", "hidden_sc", "y", "row_token"]
     assert [c["name"] for c in gemm["channels"] if c["optional"]] == ["row_token"]
     assert {t["name"]: t["bytes"] for t in gemm["provider"]["abi_types"]} == {"MokGemmResidue": 264, "MokMxView": 48}
-    assert [s["id"] for s in HOST["scalars"]] == [1, 2, 3, 4, 10, 11, 12, 60, 61, 62, 63, 64]
+    assert [s["id"] for s in HOST["scalars"]] == [1, 2, 3, 4, 10, 11, 12, 60, 61, 62, 63, 64, 65]
+    assert [c["name"] for c in GROUPS["mok.framework"]["channels"]] == ["tokens_per_expert", "workspace"]
     assert broker.evaluate_extents("mok.num_local_experts, floor(mok.hidden,64), ceil(mok.intermediate, 128), 4", SCALARS) == (4, 5, 2, 4)
     with pytest.raises(PlkError):
         broker.evaluate_extents("mok.hidden * 2", SCALARS)
@@ -222,7 +238,7 @@ def test_launch_verb_takes_a_host_link_through_its_providers(tmp_path):
     from pipelink_amd.pipec.clauses import LaunchError
     from pipelink_amd.host.fixture import Fixture, load_inputs
 
-    link_path = os.path.join(ROOT, "pipelink_amd", "stages", "mok", "build", "link", "link.json")
+    link_path = _LINK_JSON
     with pytest.raises(LaunchError) as err:
         launcher.launch(link_path, grid=(8,))
     assert err.value.failures[0].path == "launch.host"                        # host-less arguments on a host link

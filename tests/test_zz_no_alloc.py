@@ -1,6 +1,7 @@
 """The entry point that allocates nothing (plk_mok_forward_static), called through the C ABI: its outputs equal
 plk_mok_forward's byte for byte on two calls in a row, the second with a smaller input (the library's fixed device
-area still holds the first call's params images then)."""
+area still holds the first call's params images and workspace then).  The first problem's rows of hidden_q are whole
+cache lines (one launch, readiness counters in the fixed area), the second's are not (two launches)."""
 import json
 
 import pytest
@@ -9,7 +10,7 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-def _device_problem(sess, inp, H, I):
+def _device_problem(sess, inp, H, I, pitch_i=None):
     from pipelink_amd.host.mok import scale_pitch, weight_codes_to_k64_tiled, weight_scales_to_slot_major
 
     dev = torch.device("cuda:0")
@@ -21,7 +22,7 @@ def _device_problem(sess, inp, H, I):
     d["w_up_q"] = weight_codes_to_k64_tiled(d["w_up_q"], H)
     d["w_down_q"] = weight_codes_to_k64_tiled(d["w_down_q"], I)
     rows = int(inp.tokens_per_expert.sum())
-    out = dict(hidden_q=torch.empty((rows, I), dtype=torch.uint8, device=dev),
+    out = dict(hidden_q=torch.empty((rows, pitch_i or I), dtype=torch.uint8, device=dev),
                hidden_sc=torch.empty((rows, scale_pitch(I)), dtype=torch.uint8, device=dev),
                y=torch.empty((rows, H), dtype=torch.bfloat16, device=dev))
     return sess.problem(**out, **d), out, d  # d keeps the input tensors alive
@@ -45,12 +46,12 @@ def test_static_entry_point_matches_forward_on_two_calls_in_a_row():
 
     paths = mok_build.images()
     link = json.loads(paths["link_json"].read_text())
-    shapes = [(700, 448, 704, 6, 2, 21), (96, 256, 320, 8, 2, 22)]  # T, H, I, E, top_k, seed: the second is smaller
+    shapes = [(700, 448, 704, 6, 2, 21, 768), (96, 256, 320, 8, 2, 22, None)]  # T, H, I, E, top_k, seed, pitch of hidden_q
     with MoKSession(paths["linked"].read_bytes(), link) as sess:
         cases = []
-        for T, H, I, E, k, seed in shapes:
+        for T, H, I, E, k, seed, pitch in shapes:
             inp = mok_inputs.generate(T, H, I, E, k, seed=seed)
-            cases.append(_device_problem(sess, inp, H, I))
+            cases.append(_device_problem(sess, inp, H, I, pitch))
         expected = []
         for prob, out, _ in cases:
             _poison(out)
@@ -61,6 +62,7 @@ def test_static_entry_point_matches_forward_on_two_calls_in_a_row():
         torch.cuda.synchronize()
         for prob, out, _ in cases:  # back to back on one stream, no host wait between them
             sess.forward_static(prob)
+        assert sess.status() == 0
         for (prob, out, _), want in zip(cases, expected):
             got = _snapshot(out)
             for g, w in zip(got, want):
@@ -68,7 +70,7 @@ def test_static_entry_point_matches_forward_on_two_calls_in_a_row():
             assert not torch.isnan(out["y"].float()).any()
 
 
-def test_static_entry_point_rejects_an_image_beyond_its_area():
+def test_static_entry_point_rejects_sizes_beyond_its_area():
     from ctypes import sizeof
 
     from pipelink_amd.host import mok_inputs
