@@ -39,9 +39,6 @@ __device__ __forceinline__ float min_raw(float a, float b) {
 
 template <bool CLAMPED>
 __device__ __forceinline__ float swiglu(float gate, float up, float limit) {
-#ifdef EXP_NOEPI
-  return gate + up;
-#endif
   if (CLAMPED) {
     gate = min_raw(gate, limit);
     up = __builtin_amdgcn_fmed3f(up, -limit, limit);
@@ -87,12 +84,13 @@ __device__ __forceinline__ void forward(const MokActResidue& p, const MokActTask
 #pragma unroll
     for (int b = 0; b < XFRAGS; ++b) {
       const int trow = xrow0(wave, b) + (lane & 31);
+      const v16f gate = from_acc(acc.v[a][b]), up = from_acc(acc.v[a + 2][b]);
       float h[16];
       float amax = 0.0f;
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
-        h[r] = swiglu<CLAMPED>(acc.v[a][b][r], acc.v[a + 2][b][r], p.swiglu_limit);
-        h[r + 1] = swiglu<CLAMPED>(acc.v[a][b][r + 1], acc.v[a + 2][b][r + 1], p.swiglu_limit);
+        h[r] = swiglu<CLAMPED>(gate[r], up[r], p.swiglu_limit);
+        h[r + 1] = swiglu<CLAMPED>(gate[r + 1], up[r + 1], p.swiglu_limit);
         amax = fmaxf(fmaxf(amax, fabsf(h[r])), fabsf(h[r + 1]));
       }
       // the other 16 columns of this row's block live in lane ^ 32

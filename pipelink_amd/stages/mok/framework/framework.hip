@@ -149,12 +149,6 @@ extern "C" __device__ void mok_framework_worker(const void* params, unsigned var
     if (!pipelink_call_gemm_ready(&view, &task, &counters)) pipelink_call_gemm_wait(&view, &task, &counters);
     mok::GemmCarry carry;
     pipelink_call_gemm_prefetch(&view, &task, &carry);
-#ifdef EXP_STAMP
-    int exp_tile = 0;
-    const MokGemmResidue* exp_g = reinterpret_cast<const MokGemmResidue*>(static_cast<const unsigned char*>(params) + EXP_STAMP);
-    unsigned long long* exp_stamps = reinterpret_cast<unsigned long long*>(exp_g->y + (size_t)exp_g->hidden.rows * exp_g->ld_y) + (size_t)blockIdx.x * 384;
-    unsigned long long s4 = wall_clock64();
-#endif
     for (;;) {
       i += turn;
       const bool has_next = i < items;
@@ -162,39 +156,17 @@ extern "C" __device__ void mok_framework_worker(const void* params, unsigned var
       if (has_next) next = sched.decode(q, i, cursor);
       else next.op = 0;  // no task: mok_gemm_fwd looks ahead to nothing
       mok::AccFrag acc;
-#ifdef EXP_STAMP
-      const unsigned long long s0 = wall_clock64();
-#endif
       pipelink_call_gemm_fwd(&view, &task, &counters, &phase, &acc, &carry, &next);
-#ifdef EXP_STAMP
-      const unsigned long long s1 = wall_clock64();
-#endif
       // The next tile's first loads fly while this tile's epilogue computes -- unless its rows are not complete yet:
       // then this tile is finished (and counted) first, so that nobody waits for a workgroup that waits.
       const bool early = has_next && pipelink_call_gemm_ready(&view, &next, &counters);
       if (early) pipelink_call_gemm_prefetch(&view, &next, &carry);
-#ifdef EXP_STAMP
-      const unsigned long long s2 = wall_clock64();
-#endif
       if (task.op == MOK_GEMM_FWD_ROUTED_GATE_UP) {
         const MokActTask act{MOK_ACT_FWD_ROUTED, task.row_begin, task.row_end, task.col_begin, task.task_idx, task.counter_idx, 0u};
         pipelink_call_act_fwd(&view, &act, &counters, &phase, &acc);
       } else {
         pipelink_call_gemm_store(&view, &task, &acc);
       }
-#ifdef EXP_STAMP
-      {
-        const unsigned long long s3 = wall_clock64();
-        if (threadIdx.x == 0 && exp_tile < 64) {
-          int rows = task.row_end - task.row_begin; rows = rows > 256 ? 256 : rows;
-          exp_stamps[exp_tile * 6 + 0] = s0; exp_stamps[exp_tile * 6 + 1] = s1; exp_stamps[exp_tile * 6 + 2] = s2;
-          exp_stamps[exp_tile * 6 + 3] = s3; exp_stamps[exp_tile * 6 + 4] = (unsigned)((rows + 31) / 32) | (unsigned)task.op << 8 | (early ? 1u << 16 : 0u);
-          exp_stamps[exp_tile * 6 + 5] = s4;
-        }
-        ++exp_tile;
-        s4 = s3;
-      }
-#endif
       if (!has_next) break;
       if (!early) {
         pipelink_call_gemm_wait(&view, &next, &counters);

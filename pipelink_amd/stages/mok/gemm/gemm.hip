@@ -70,9 +70,7 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
 }
 // 16 (4) bytes per lane, buffer -> LDS; lane i lands at lds + 16*i (4*i)
 __device__ __forceinline__ void buf16_to_lds(rsrc_t r, uint32_t lane_off, uint32_t uni_off, unsigned char* lds) {
-#ifndef EXP_NOLOADS
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lptr_t)lds, 16, (int)lane_off, (int)uni_off, 0, 0);
-#endif
 }
 __device__ __forceinline__ void buf4_to_lds(rsrc_t r, uint32_t lane_off, uint32_t uni_off, unsigned char* lds) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lptr_t)lds, 4, (int)lane_off, (int)uni_off, 0, 0);
@@ -82,11 +80,7 @@ __device__ __forceinline__ void buf4_to_lds(rsrc_t r, uint32_t lane_off, uint32_
 // line can hold both finished and unfinished parts: the scale rows of `hidden` (a line spans rows of different row
 // tiles) and the readiness counters.
 __device__ __forceinline__ void buf16_to_lds_device_scope(rsrc_t r, uint32_t lane_off, uint32_t uni_off, unsigned char* lds) {
-#ifdef EXP_NO_SC1_XSC
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lptr_t)lds, 16, (int)lane_off, (int)uni_off, 0, 0);
-#else
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lptr_t)lds, 16, (int)lane_off, (int)uni_off, 0, 16);
-#endif
 }
 __device__ __forceinline__ void buf4_to_lds_device_scope(rsrc_t r, uint32_t lane_off, uint32_t uni_off, unsigned char* lds) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lptr_t)lds, 4, (int)lane_off, (int)uni_off, 0, 16);
@@ -214,13 +208,8 @@ __device__ __forceinline__ void issue_one(const Loader& ld, const Rings<DEPTH>& 
 // (measured on gfx950 with a one-instruction probe).  So a lane reads chunks half and
 // half + 2 of its row; with the XOR swizzle the second is the first with bit 5 flipped.
 __device__ __forceinline__ v8i read_frag(const unsigned char* slot, int off) {
-#ifdef EXP_NOREADS
-  v4i lo = {off, off + 1, off + 2, off + 3}, hi = {off + 4, off + 5, off + 6, off + 7};
-  asm volatile("" : "+v"(lo), "+v"(hi));
-#else
   const v4i lo = *reinterpret_cast<const v4i*>(slot + off);
   const v4i hi = *reinterpret_cast<const v4i*>(slot + (off ^ 32));
-#endif
   v8i r;
   r.s0 = lo.x; r.s1 = lo.y; r.s2 = lo.z; r.s3 = lo.w;
   r.s4 = hi.x; r.s5 = hi.y; r.s6 = hi.z; r.s7 = hi.w;
@@ -306,12 +295,8 @@ __device__ __forceinline__ void mma_step(const Operands& o, const int (&sx)[XFRA
   for (int a = 0; a < WFRAGS; ++a)
 #pragma unroll
     for (int b = 0; b < XFRAGS; ++b)
-#ifndef EXP_NOMFMA
       acc.v[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.w[a], o.x[b], acc.v[a][b], 0, 0, ODD ? 2 : 0,
                                                                     sw[a], ODD ? 2 : 0, sx[b]);
-#else
-      asm volatile("" :: "v"(o.w[a]), "v"(o.x[b]), "v"(sw[a]), "v"(sx[b]));
-#endif
 }
 
 // Looking ahead.  While a tile is multiplied the framework names the task that comes after it; `stage` asks memory
@@ -363,11 +348,10 @@ __device__ __forceinline__ void wait_rows(const MokGemmTask& t, const MokCounter
   __syncthreads();
 }
 
-// The two operands of a task as this wave sees them, copied out of the residue in one go: a field fetched where it is
-// used is a scalar load and a wait of its own.
+// The two operands of a task as this wave sees them.
 struct Views {
-  MokMxView act;  // routed rows: x (gate/up op) or hidden (down op)
-  MokMxView w;    // weight rows this wave loads: gate or up (by wave) or down
+  const MokMxView& act;  // routed rows: x (gate/up op) or hidden (down op)
+  const MokMxView& w;    // weight rows this wave loads: gate or up (by wave) or down
 };
 __device__ __forceinline__ Views views_of(const MokGemmResidue& g, const MokGemmTask& t) {
   const int wave = __builtin_amdgcn_readfirstlane(fresh_tid() >> 6);
@@ -412,11 +396,7 @@ __device__ __forceinline__ Loader make_loader(const Views& v, const MokGemmTask&
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: resources chosen by it stay scalar
   const bool gate_up = t.op == MOK_GEMM_FWD_ROUTED_GATE_UP;
-#ifdef EXP_SAMEW
-  const int expert = 0;
-#else
   const int expert = __builtin_amdgcn_readfirstlane(t.expert);
-#endif
   const MokMxView& act = v.act;
   Loader ld;
   const int lrow = lane >> 2;
@@ -432,11 +412,7 @@ __device__ __forceinline__ Loader make_loader(const Views& v, const MokGemmTask&
 #pragma unroll
   for (int i = 0; i < W_GROUPS; ++i) {
     const int wl = (wave * W_GROUPS + i) * 16 + lrow;  // tile-local weight row
-#ifdef EXP_SAMEW
-    const int col = (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
-#else
     const int col = t.col_begin + (gate_up ? (wl & (TILE_W / 2 - 1)) : wl);
-#endif
     ld.wsrc[i] = col < wv.rows ? (uint32_t)col * (uint32_t)K_SLOT + chunk : PAST_THE_END;  // weights are K-tiled: [K/64][rows][64]
   }
   ld.w = make_rsrc(wv.q + (int64_t)expert * wv.expert_pitch_q, (uint32_t)wv.rows * (uint32_t)wv.k);
@@ -561,9 +537,7 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   // The look-ahead loads go here, behind the prologue's: the waits below count the loads that may still be in flight
   // behind the slot they need, and loads return in order, so one or two more of the youngest only make the next few
   // waits ask for as many more of the oldest.
-#ifndef EXP_NO_STAGE
   if (upcoming->op != 0) stage(g, *upcoming, counters);
-#endif
   wait_loads_and_reads_dyn(loads_younger_than_slot<DEPTH>(0, -1, n));
   wg_barrier();
   auto xnext = [](int b, int by) {  // (b + by) mod XDEPTH for 0 <= b < XDEPTH, 0 <= by <= XDEPTH
@@ -636,12 +610,8 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       auto place = [&](auto I_) {
         constexpr int I = decltype(I_)::value;
         constexpr int A = I / XFRAGS, B = I % XFRAGS;
-#ifndef EXP_NOMFMA
         acc.v[A][B] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cur.w[A], cur.x[B], acc.v[A][B], 0, 0, ODD ? 2 : 0,
                                                                       sw[A], ODD ? 2 : 0, sx[B]);
-#else
-        asm volatile("" :: "v"(cur.w[A]), "v"(cur.x[B]), "v"(sw[A]), "v"(sx[B]));
-#endif
         __builtin_amdgcn_sched_barrier(0);  // the MFMA goes first: the pipe is what must not wait
         if constexpr (I == 1) {
           wait_loads_and_reads<ODD ? STEADY_ODD : STEADY_EVEN>();
@@ -757,13 +727,14 @@ __device__ __forceinline__ void store_down(const MokGemmResidue& g, const MokGem
       const int row = t.row_begin + xrow0(wave, b) + (lane & 31);
 #pragma unroll
       for (int a = 0; a < WFRAGS; ++a) {
+        const v16f f = from_acc(acc.v[a][b]);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int col = t.col_begin + wrow0(wave, a) + 8 * q + 4 * (lane >> 5);
           if (row < t.row_end && col < g.w_down.rows) {
             uint2 pk;
-            pk.x = pack_bf16x2(acc.v[a][b][4 * q + 0], acc.v[a][b][4 * q + 1]);
-            pk.y = pack_bf16x2(acc.v[a][b][4 * q + 2], acc.v[a][b][4 * q + 3]);
+            pk.x = pack_bf16x2(f[4 * q + 0], f[4 * q + 1]);
+            pk.y = pack_bf16x2(f[4 * q + 2], f[4 * q + 3]);
             *reinterpret_cast<uint2*>(g.y + (int64_t)row * g.ld_y + col) = pk;
           }
         }
@@ -783,12 +754,13 @@ __device__ __forceinline__ void store_down(const MokGemmResidue& g, const MokGem
           unsigned char* rowp = stage + (xrow0(wave, b) - pass * ROWS + (lane & 31)) * Y_PITCH;
 #pragma unroll
           for (int a = 0; a < WFRAGS; ++a) {
+            const v16f f = from_acc(acc.v[a][b]);
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               const int col = wrow0(wave, a) + 8 * q + 4 * (lane >> 5);
               uint2 pk;
-              pk.x = pack_bf16x2(acc.v[a][b][4 * q + 0], acc.v[a][b][4 * q + 1]);
-              pk.y = pack_bf16x2(acc.v[a][b][4 * q + 2], acc.v[a][b][4 * q + 3]);
+              pk.x = pack_bf16x2(f[4 * q + 0], f[4 * q + 1]);
+              pk.y = pack_bf16x2(f[4 * q + 2], f[4 * q + 3]);
               *reinterpret_cast<uint2*>(rowp + col * 2) = pk;
             }
           }
@@ -846,13 +818,8 @@ extern "C" __device__ void mok_gemm_wait(const void* view, const MokGemmTask* ta
 extern "C" __device__ void mok_gemm_prefetch(const void* view, const MokGemmTask* task, mok::GemmCarry* carry) {
   const auto& g = mok_gemm_residue(view);
   switch (pipelink_mok_gemm_depth()) {  // a link-time constant: one case survives
-#ifdef EXP_NO_STAGE
-    case 2: mok_gemm_owner::prefetch<2>(g, *task, *carry, false); break;
-    default: mok_gemm_owner::prefetch<4>(g, *task, *carry, false); break;
-#else
     case 2: mok_gemm_owner::prefetch<2>(g, *task, *carry, true); break;
     default: mok_gemm_owner::prefetch<4>(g, *task, *carry, true); break;
-#endif
   }
 }
 

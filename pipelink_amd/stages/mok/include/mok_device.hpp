@@ -38,6 +38,15 @@ struct AccFrag {
   v16f v[WFRAGS][XFRAGS];
 };
 
+// One fragment of the accumulator, which stays in the accumulator registers up to here.  An epilogue takes each
+// fragment through this where it starts to use it: the compiler may otherwise copy the whole tile to vector
+// registers as soon as the mainloop is over, ahead of the next tile's prefetch, which leaves that code short of
+// registers (its spills then wait for the prefetch's loads, because every wait on a scratch load does).
+__device__ __forceinline__ v16f from_acc(v16f v) {
+  asm volatile("" : "+a"(v));
+  return v;
+}
+
 // What the GEMM owner's prefetch export hands to its forward export for the same tile: the
 // lane's gathered routed-row offsets (they cost a dependent global load, which the prefetch
 // takes off the forward call's critical path).  Opaque to the other stages.

@@ -32,16 +32,18 @@ def test_link_json_records_the_solved_cell(cell):
     out, res = cell
     link = json.loads((out / "link" / "link.json").read_text())
     assert link["kernel_symbol"] == "pipelink_kernel" and link["threads"] == 256
-    # four 16 KB weight buffers, five 16 KB routed-row buffers, 12 KB of scale buffers + the schedule table fit 160 KB of LDS: the preferred depth is taken
+    # four 16 KB weight buffers, five 16 KB routed-row buffers, 12 KB of scale buffers, the staged task's 1280 bytes + the schedule table fit 160 KB of LDS: the preferred depth is taken
     assert link["bindings"]["pipelink_mok_gemm_depth"] == [4, "solved"]
-    # head (4 buffers + 12 KB of scale buffers, whole kernel) + arena (5 buffers, GEMM phase) + schedule table
-    assert link["dyn_smem_bytes"] == (4 * 16384 + 12288) + 5 * 16384 + 2056 <= 160 * 1024
+    # head (4 buffers + 12 KB of scale buffers + the staged task's row tokens and counter copy, whole kernel)
+    # + arena (5 buffers, GEMM phase) + schedule table (two prefix-sum tables of 257 entries + the "last workgroup" flag)
+    assert link["dyn_smem_bytes"] == (4 * 16384 + 12288 + 1024 + 256) + 5 * 16384 + (2 * 257 * 4 + 8) <= 160 * 1024
     assert link["bindings"]["pipelink_mok_act_arena"][0] == link["bindings"]["pipelink_mok_gemm_arena"][0]  # phase-exclusive
     assert [e["stage_id"] for e in link["params"]["entries"]] == ["mok.framework", "mok.gemm", "mok.act"]
-    assert link["params"]["total_bytes"] == 344
-    assert {e["channel"] for e in link["protocol_expansions"]} == {"gemm_init", "gemm_prefetch", "gemm_fwd", "gemm_store", "act_init", "act_fwd"}
+    assert link["params"]["total_bytes"] == 32 + 264 + 40
+    assert {e["channel"] for e in link["protocol_expansions"]} == {"gemm_init", "gemm_fini", "gemm_stage", "gemm_ready", "gemm_wait", "gemm_prefetch",
+                                                                   "gemm_fwd", "gemm_store", "act_init", "act_fwd"}
     obs = link["observed"]
-    assert obs["calls"] == 0 and obs["private_segment_fixed_size"] <= 256 and obs["mfma"] >= 16   # a few dwords spilled in the tile set-up at most
+    assert obs["calls"] == 0 and obs["private_segment_fixed_size"] <= 64 and obs["mfma"] >= 16   # a few dwords spilled in the tile set-up at most
     assert obs["vgpr_count"] <= link["regs_cap"] == 512
     assert link["facts"]["mok.gemm.TILE_X"] == 256
     assert set(link["input_hashes"]) == {"mok.framework", "mok.gemm", "mok.act"}
@@ -176,11 +178,11 @@ def test_hostless_launcher_params_contract(cell):
     def params(addr):
         seen.update(addr)
         assert be.log.count("upload") == 1      # every buffer is in place before params() runs
-        return {"mok.framework": b"\x01" * 40, "mok.gemm": b"\x02" * 264, "mok.act": b"\x03" * 40}
+        return {"mok.framework": b"\x01" * 32, "mok.gemm": b"\x02" * 264, "mok.act": b"\x03" * 40}
     s = open_hostless(link, buffers={"a": np.arange(4, dtype=np.int32), "b": ((8,), np.float32)}, params=params,
                       grid=(16,), backend=be, image=image)
     blob = be.mem[s.params_addr]
-    assert blob[0:40] == b"\x01" * 40 and blob[40:304] == b"\x02" * 264 and blob[304:344] == b"\x03" * 40
+    assert blob[0:32] == b"\x01" * 32 and blob[32:296] == b"\x02" * 264 and blob[296:336] == b"\x03" * 40
     s.launch()
     assert be.launches == [(s.params_addr, (16, 1, 1), (256, 1, 1), link["dyn_smem_bytes"])]
     assert s.read("a").tolist() == [0, 1, 2, 3] and s.read("b").tolist() == [0.0] * 8
