@@ -6,10 +6,11 @@ One step = one forward over the whole batch: T=8192 tokens, d_model=d_ff=2880, 3
 top-4 routing (32768 routed rows), inputs already resident in HBM.  Prints ONE JSON line:
 metric = MXFP8 grouped-GEMM TFLOP/s on the algorithmic (unpadded) flop count
 2*R*H*I*3 = 1.6307e12 per forward (weights in the layouts the kernel streams: K-tiled codes, slot-major scales), plus
-  roofline      -- the gate/up pass (the dominant kernel) timed with HIP events on its launch
-                   stream, against the 5.0 PFLOP/s dense FP8 MFMA peak;
+  roofline      -- the forward's one kernel (both grouped GEMMs in one launch), its launch duration measured with HIP
+                   events on its launch stream over the timed steps, against the 5.0 PFLOP/s dense FP8 MFMA peak; the
+                   two GEMMs launched separately (the library's other mode) are timed beside it;
   cpu_baseline  -- the CPU oracle (torch fp32 dequant-then-matmul) timed on the host cores on
-                   the first 1024 tokens of the same inputs;
+                   the whole batch of the same inputs, and on its first 1024 tokens;
   linked_over_one_unit -- paired ABBA/BAAB timing of the linked image against the one-unit
                    control (evaluator/harness/parity/example.py:104-166 in the reference);
   power         -- board power and shader clock the driver reports (hwmon power1_input,
@@ -39,9 +40,34 @@ FLOPS_GATE_UP = 2.0 * T * TOPK * H * I * 2
 FLOPS_DOWN = 2.0 * T * TOPK * I * H
 FLOPS_TOTAL = FLOPS_GATE_UP + FLOPS_DOWN
 PEAK_FP8_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
-# HBM-side bytes of one gate/up launch: FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this script, each
-# scaled by what the same counter reads for a 1 GiB device copy (--copy-calibration): 2.0 and 1.0 KiB per unit.
-TRAFFIC_GATE_UP_BYTES = 1.105e9
+# HBM-side bytes of one launch of the forward's kernel: FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this
+# script, each scaled by what the same counter reads for a 1 GiB device copy (--copy-calibration).  The figures are
+# kept in a JSON file next to the profile summary they come from; without the file `traffic` is null.
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "pipelink_kernel_bench_shape_traffic.json")
+TILE = 256  # the kernel's tile: 256 routed rows x 256 weight rows (gate/up: 128 gate + 128 up columns)
+
+
+def traffic_bytes():
+    try:
+        with open(TRAFFIC_JSON) as f:
+            return float(json.load(f)["traffic_bytes_per_launch"])
+    except (OSError, KeyError, ValueError):
+        return None
+
+
+def executed_flops(counts):
+    """Flops the kernel's waves execute for these per-expert row counts: a wave multiplies its 128 x 128 share of a
+    tile over the whole contraction unless the share starts past the expert's last row or past the last output
+    column (then it only loads).  Shares that are partly past the end are multiplied in full."""
+    total = 0.0
+    for c in counts:
+        for first in range(0, int(c), TILE):
+            row_waves = 1 if int(c) - first <= TILE // 2 else 2
+            for cols, k, step in ((I, H, TILE // 2), (H, I, TILE)):  # gate/up (per matrix), down
+                for col_begin in range(0, cols, step):
+                    col_waves = sum(col_begin + w * 64 < cols for w in (0, 1))
+                    total += row_waves * col_waves * 128 * 128 * 2.0 * k
+    return total
 
 
 def make_inputs(dev, seed=0):
@@ -81,7 +107,7 @@ def make_inputs(dev, seed=0):
 
 class PowerSampler:
     """Reads board power (hwmon power1_input, microwatts) and the current shader clock level
-    (pp_dpm_sclk, the line marked with *) every 50 ms on a thread; best effort: a box that
+    (pp_dpm_sclk, the line marked with *) every 10 ms on a thread; best effort: a box that
     does not expose them yields nulls."""
 
     def __init__(self):
@@ -111,7 +137,7 @@ class PowerSampler:
             m = re.search(r"(\d+)\s*Mhz\s*\*", c or "", re.IGNORECASE)
             if m:
                 self.mhz.append(int(m.group(1)))
-            self._stop.wait(0.05)
+            self._stop.wait(0.01)
 
     def __enter__(self):
         self._thread = threading.Thread(target=self._run, daemon=True)
@@ -128,16 +154,24 @@ class PowerSampler:
                 "draw_w": round(statistics.median(self.watts), 1) if self.watts else None,
                 "sclk_mhz": round(statistics.median(self.mhz)) if self.mhz else None,
                 "samples": len(self.watts),
-                "source": "hwmon power1_input / power1_cap, pp_dpm_sclk, sampled every 50 ms during the timed steps"}
+                "source": "hwmon power1_input / power1_cap, pp_dpm_sclk, sampled every 10 ms while the forward runs back to back: "
+                          "during the timed steps and, where those are too few for 10 samples, during untimed ones after them"}
 
 
 def mfma_ceiling(be, torch, seconds=1.0):
     """What back-to-back v_mfma_scale_f32_32x32x64_f8f6f4 alone sustain on this board (one wave per
     SIMD, operands in registers, no LDS or memory traffic): with random e4m3 operands the board
     sits at its power limit and clocks down; with zero operands it runs at the full clock."""
-    from pipelink_amd.host.backend import check, load_library
+    import ctypes
 
-    lib = load_library()
+    path = os.path.join(ROOT, "pipelink_amd", "libplk_bench_probe.so")  # built by __graft_entry__.build()
+    lib = ctypes.CDLL(path)
+    lib.plk_probe_mfma_fp8.restype = ctypes.c_int
+    lib.plk_probe_mfma_fp8.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint64, ctypes.c_void_p]
+
+    def check(status):
+        if status != 0:
+            raise RuntimeError(f"plk_probe_mfma_fp8 failed with status {status}")
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     sink = torch.zeros(16, dtype=torch.float32, device="cuda:0")
     stream = torch.cuda.current_stream().cuda_stream
@@ -147,7 +181,7 @@ def mfma_ceiling(be, torch, seconds=1.0):
     for name, zero in (("random_operands", 0), ("zero_operands", 1)):
         def batch():
             for _ in range(per_batch):
-                check(lib, lib.plk_probe_mfma_fp8(cus, iters, zero, sink.data_ptr(), stream))
+                check(lib.plk_probe_mfma_fp8(cus, iters, zero, sink.data_ptr(), stream))
         end = time.perf_counter() + seconds  # clock / power ramp
         while time.perf_counter() < end:
             batch()
@@ -174,35 +208,40 @@ def mfma_ceiling(be, torch, seconds=1.0):
     return out
 
 
-def cpu_baseline(inp, row_major, sample_tokens=1024, reps=3):
-    """The oracle on the host cores, first `sample_tokens` tokens of the same inputs."""
-    import numpy as np
+def cpu_baseline(inp, row_major, slice_tokens=1024):
+    """The oracle on the host cores: the whole batch of the same inputs (one run after one warm-up), and its first
+    `slice_tokens` tokens (median of 3 after a warm-up)."""
     import torch
     from oracle import moe_ffn
     from pipelink_amd.host import mok_inputs
 
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    g = torch.Generator().manual_seed(0)
-    logits = torch.randn(T, E, generator=g)[:sample_tokens]
-    counts, row_token = mok_inputs.route(logits, TOPK)
     host = {k: v.cpu() for k, v in {**inp, **row_major}.items()}
-    args = dict(x_q=host["x_q"][:sample_tokens, :H], x_sc=host["x_sc"][:sample_tokens],
-                wg_q=host["w_gate_q"][:, :, :H], wg_sc=host["w_gate_sc"], wu_q=host["w_up_q"][:, :, :H],
-                wu_sc=host["w_up_sc"], wd_q=host["w_down_q"][:, :, :I], wd_sc=host["w_down_sc"], counts=counts,
-                row_token=row_token)
-    times = []
-    for rep in range(reps + 1):
-        t0 = time.perf_counter()
-        moe_ffn.moe_ffn_forward_torch(**args)
-        if rep:
-            times.append(time.perf_counter() - t0)
-    sec = statistics.median(times)
-    flops = FLOPS_TOTAL * sample_tokens / T
-    return {"value": round(flops / sec / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"first {sample_tokens} of {T} tokens (all {E} experts' weights dequantised inside the timed "
-                      f"region), median of {reps} runs after 1 warm-up, {sec * 1e3:.0f} ms per forward, "
-                      f"torch {torch.__version__} fp32"}
+
+    def timed(tokens, reps):
+        g = torch.Generator().manual_seed(0)
+        logits = torch.randn(T, E, generator=g)[:tokens]
+        counts, row_token = mok_inputs.route(logits, TOPK)
+        args = dict(x_q=host["x_q"][:tokens, :H], x_sc=host["x_sc"][:tokens],
+                    wg_q=host["w_gate_q"][:, :, :H], wg_sc=host["w_gate_sc"], wu_q=host["w_up_q"][:, :, :H],
+                    wu_sc=host["w_up_sc"], wd_q=host["w_down_q"][:, :, :I], wd_sc=host["w_down_sc"], counts=counts,
+                    row_token=row_token)
+        times = []
+        for rep in range(reps + 1):
+            t0 = time.perf_counter()
+            moe_ffn.moe_ffn_forward_torch(**args)
+            if rep:
+                times.append(time.perf_counter() - t0)
+        return statistics.median(times)
+
+    sec_slice = timed(slice_tokens, 3)
+    sec_full = timed(T, 1)
+    return {"value": round(FLOPS_TOTAL / sec_full / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"the whole batch ({T} tokens, {T * TOPK} routed rows; all {E} experts' weights dequantised inside the "
+                      f"timed region): one run after 1 warm-up, {sec_full * 1e3:.0f} ms per forward, torch {torch.__version__} fp32",
+            "slice": {"value": round(FLOPS_TOTAL * slice_tokens / T / sec_slice / 1e12, 4), "tokens": slice_tokens,
+                      "ms_per_forward": round(sec_slice * 1e3), "runs": "median of 3 after 1 warm-up"}}
 
 
 def main() -> int:
@@ -260,12 +299,27 @@ def main() -> int:
     for _ in range(args.warmup):
         linked.forward(prob)
     torch.cuda.synchronize()
+    e0, e1 = be.event_create(), be.event_create()
     with PowerSampler() as power:
         t0 = time.perf_counter()
+        be.event_record(e0)
         for _ in range(args.steps):
             linked.forward(prob)
+        be.event_record(e1)
         torch.cuda.synchronize()
         ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+        # the forward is one launch: the events bracket `steps` launches that run back to back on the launch stream
+        ms_launch = be.event_elapsed_time(e0, e1) / args.steps
+        while 0 < len(power.watts) < 10:  # too few timed steps for ten readings: go on, untimed
+            for _ in range(20):
+                linked.forward(prob)
+            torch.cuda.synchronize()
+    be.event_destroy(e0)
+    be.event_destroy(e1)
+    status = linked.status()
+    if status != 0:
+        print(f"bench.py: the forward raised status {status} (a tile gave up waiting for its rows)", file=sys.stderr)
+        return 1
 
     def event_ms(sess, which, n):
         e0, e1 = be.event_create(), be.event_create()
@@ -279,9 +333,9 @@ def main() -> int:
         be.event_destroy(e1)
         return ms
 
-    # per-pass launch durations: the forward is launched as its two passes in turn, as above, and
-    # each pass is bracketed by its own pair of events (a loop over one pass alone would keep that
-    # pass's weights in the last-level cache and change the clock the other pass leaves it)
+    # the library's other mode, one launch per GEMM: the two passes in turn, each bracketed by its own pair of
+    # events (a loop over one pass alone would keep that pass's weights in the last-level cache and change
+    # the clock the other pass leaves it)
     n = min(max(args.steps, 10), 200)
     ev = [[be.event_create() for _ in range(3)] for _ in range(n)]
     for a, b, c in ev:
@@ -330,11 +384,16 @@ def main() -> int:
                    "experts": E, "top_k": TOPK, "routed_rows": rows, "image": "linked",
                    "pct_of_fp8_mfma_peak": round(FLOPS_TOTAL / (ms_per_step * 1e-3) / 1e12 / PEAK_FP8_TFLOPS * 100, 2),
                    "ms_per_token": round(ms_per_step / T, 7)},
-        "roofline": {"bound": "mfma", "kernel": "pipelink_kernel (gate/up pass: grouped GEMM + SwiGLU + requant)",
-                     "achieved": round(FLOPS_GATE_UP / (ms_gate_up * 1e-3) / 1e12, 2), "peak": PEAK_FP8_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(FLOPS_GATE_UP / (ms_gate_up * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4),
-                     "traffic": TRAFFIC_GATE_UP_BYTES, "launch_ms": round(ms_gate_up, 4),
-                     "down_pass": {"achieved": round(FLOPS_DOWN / (ms_down * 1e-3) / 1e12, 2), "launch_ms": round(ms_down, 4)}},
+        "roofline": {"bound": "mfma",
+                     "kernel": "pipelink_kernel (one launch: gate/up grouped GEMM + SwiGLU + requant tiles, then down grouped "
+                               "GEMM tiles that wait for their rows' readiness counters)",
+                     "achieved": round(FLOPS_TOTAL / (ms_launch * 1e-3) / 1e12, 2), "peak": PEAK_FP8_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(FLOPS_TOTAL / (ms_launch * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4),
+                     "traffic": traffic_bytes(), "launch_ms": round(ms_launch, 4),
+                     "executed_over_algorithmic_flops": round(executed_flops(inp["tokens_per_expert"].tolist()) / FLOPS_TOTAL, 4),
+                     "two_launches": {
+                         "gate_up_pass": {"achieved": round(FLOPS_GATE_UP / (ms_gate_up * 1e-3) / 1e12, 2), "launch_ms": round(ms_gate_up, 4)},
+                         "down_pass": {"achieved": round(FLOPS_DOWN / (ms_down * 1e-3) / 1e12, 2), "launch_ms": round(ms_down, 4)}}},
         "linked_over_one_unit": pair,
         "power": power.report(),
     }
@@ -343,11 +402,11 @@ def main() -> int:
         # the published peak is 256 CUs x 4 SIMDs x 2048 FP8 flop per clock at 2.4 GHz
         at_clock = PEAK_FP8_TFLOPS * sclk / 2400.0
         out["roofline"]["peak_at_reported_sclk"] = round(at_clock, 1)
-        out["roofline"]["frac_at_reported_sclk"] = round(FLOPS_GATE_UP / (ms_gate_up * 1e-3) / 1e12 / at_clock, 4)
+        out["roofline"]["frac_at_reported_sclk"] = round(FLOPS_TOTAL / (ms_launch * 1e-3) / 1e12 / at_clock, 4)
     if ceiling:
         out["mfma_ceiling"] = ceiling
         rnd = ceiling["random_operands"]["tflops"]
-        out["roofline"]["frac_of_measured_mfma_ceiling"] = round(FLOPS_GATE_UP / (ms_gate_up * 1e-3) / 1e12 / rnd, 4)
+        out["roofline"]["frac_of_measured_mfma_ceiling"] = round(FLOPS_TOTAL / (ms_launch * 1e-3) / 1e12 / rnd, 4)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(inp, row_major)
     print(json.dumps(out))

@@ -88,14 +88,6 @@ int plk_hip_module_function(plk_hip_module* module, const char* name, uint32_t d
 int plk_hip_launch(plk_hip_function* fn, const uint32_t grid[3], const uint32_t block[3], uint32_t dyn_lds_bytes,
                    void* stream, uint64_t params_addr);
 
-/* Measurement aid (no counterpart in the reference): launches `workgroups` workgroups of 256
- * threads (one wave per SIMD) that each issue iters * 16 v_mfma_scale_f32_32x32x64_f8f6f4 per wave
- * on operands held in registers -- random finite e4m3 bytes, or zeros -- and nothing else.  Timed by
- * the caller it gives what the matrix pipe alone sustains at the board's power limit:
- * flop = workgroups * 4 * iters * 16 * 131072.  `sink` is 4 bytes of device memory (never written
- * in practice). */
-int plk_probe_mfma_fp8(int32_t workgroups, int32_t iters, int32_t zero_operands, uint64_t sink, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -80,7 +80,6 @@ SIGNATURES = {
     "plk_mok_status": (c_int, [c_void_p, c_void_p, POINTER(ctypes.c_uint32)]),
     "plk_mxfp8_scales_to_slot_major": (c_int, [c_uint64, c_int64, c_int32, c_int32, c_uint64, c_void_p]),
     "plk_mxfp8_codes_to_k64_tiled": (c_int, [c_uint64, c_int64, c_int32, c_int64, c_uint64, c_void_p]),
-    "plk_probe_mfma_fp8": (c_int, [c_int32, c_int32, c_int32, c_uint64, c_void_p]),
     "plk_mxfp8_quantize": (c_int, [c_uint64, c_int, c_int64, c_int32, c_uint64, c_int32, c_uint64, c_int32, c_void_p]),
 }
 
