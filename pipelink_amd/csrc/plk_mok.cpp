@@ -341,14 +341,22 @@ __global__ void __launch_bounds__(256) mxfp8_quantize_kernel(const void* __restr
     amax = fmaxf(amax, __shfl_xor(amax, 1));
     amax = fmaxf(amax, __shfl_xor(amax, 2));
     amax = fmaxf(amax, __shfl_xor(amax, 4));
-    int e = (int)((__float_as_uint(amax) >> 23) & 0xFFu) - 8;
+    // fmaxf drops a NaN operand: a NaN anywhere in the block is carried beside the maximum, and makes the block's
+    // largest magnitude NaN (exponent field 255, like an infinity), as a maximum that propagates NaN would
+    int has_nan = (v[0] != v[0]) | (v[1] != v[1]) | (v[2] != v[2]) | (v[3] != v[3]);
+    has_nan |= __shfl_xor(has_nan, 1);
+    has_nan |= __shfl_xor(has_nan, 2);
+    has_nan |= __shfl_xor(has_nan, 4);
+    int e = (has_nan ? 255 : (int)((__float_as_uint(amax) >> 23) & 0xFFu)) - 8;
     e = e < 0 ? 0 : e;
     const float inv = __uint_as_float((uint32_t)(254 - e) << 23);
     float s[4];
-    for (int j = 0; j < 4; ++j) s[j] = fminf(fmaxf(v[j] * inv, -448.0f), 448.0f);
+    for (int j = 0; j < 4; ++j) s[j] = fminf(fmaxf(v[j] * inv, -448.0f), 448.0f);  // (a NaN becomes -448 here: replaced below)
     int pk = 0;
     pk = __builtin_amdgcn_cvt_pk_fp8_f32(s[0], s[1], pk, false);
     pk = __builtin_amdgcn_cvt_pk_fp8_f32(s[2], s[3], pk, true);
+    for (int j = 0; j < 4; ++j)  // a NaN element keeps its sign and becomes e4m3's NaN code
+      if (v[j] != v[j]) pk = (pk & ~(0xFF << (8 * j))) | (int)((0x7Fu | ((__float_as_uint(v[j]) >> 24) & 0x80u)) << (8 * j));
     *reinterpret_cast<uint32_t*>(dq + row * (int64_t)ld_q + cb * 32 + sub * 4) = (uint32_t)pk;
     if (sub == 0) dsc[row * ld_sc + cb] = (uint8_t)e;
     // zero the pad bytes of the scale row once per row

@@ -19,6 +19,8 @@ def open_session(link_json: str | Path, q_bits: np.ndarray, k_bits: np.ndarray, 
     (A link names one mask package; the params blob must be addressed to it.)"""
     if window is not None and window < 1:
         raise ValueError("a window is at least one key")
+    if scale is not None and not (np.isfinite(scale) and scale > 0):
+        raise ValueError("the softmax scale must be a positive finite number (masked scores are -1e30 times it)")
     if q_bits.ndim != 4 or k_bits.shape != v_bits.shape or k_bits.ndim != 4:
         raise ValueError("q is [B, Hq, S, D]; k and v are [B, Hkv, S, D]")
     b, hq, s, d = q_bits.shape

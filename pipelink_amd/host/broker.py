@@ -68,14 +68,14 @@ class Geometry(Structure):
                 ("cluster", Dim3), ("reserved", c_uint32), ("dynamic_smem_bytes", c_uint64)]
 
 
-class Domain(Structure):
+class DomainRecord(Structure):  # plk_domain_v2 (the caller-facing Domain tuple is the fixture module's)
     _fields_ = [("domain_id", c_uint32), ("rank", c_uint32), ("world", c_uint32), ("reserved", c_uint32)]
 
 
 class Common(Structure):
     _fields_ = [("header", Header), ("owner_id", c_uint32), ("channel_count", c_uint32), ("domain_count", c_uint32),
                 ("reserved", c_uint32), ("shared", POINTER(SharedScalars)), ("channels", POINTER(TensorMeta)),
-                ("domains", POINTER(Domain)), ("block", Dim3), ("cluster", Dim3), ("dynamic_smem_bytes", c_uint64),
+                ("domains", POINTER(DomainRecord)), ("block", Dim3), ("cluster", Dim3), ("dynamic_smem_bytes", c_uint64),
                 ("profile", ProfileDigest), ("owner_contract", Digest)]
 
 
@@ -170,7 +170,7 @@ NEUTRAL_TYPES = [
     (0x7000000E, "plk_scalar_v2", Scalar), (0x7000000F, "plk_shared_scalars_v2", SharedScalars),
     (0x70000010, "plk_transfer_report_v2", TransferReport), (0x70000011, "plk_tensor_meta_v2", TensorMeta),
     (0x70000012, "plk_workspace_demand_v2", WorkspaceDemand), (0x70000013, "plk_workspace_resource_v2", WorkspaceResource),
-    (0x70000014, "plk_domain_v2", Domain),
+    (0x70000014, "plk_domain_v2", DomainRecord),
 ]
 
 # ctypes mirrors of the owner-local record types a link may name (C name -> mirror)

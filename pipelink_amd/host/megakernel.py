@@ -14,7 +14,9 @@ def open_session(link_json: str | Path, weights: np.ndarray, kv_cache: np.ndarra
                  hkv: int, dff: int, vocab: int, pos: int, workgroups: int, backend=None, image: str | Path | None = None) -> HostlessSession:
     """weights: packed bf16 bit patterns (uint16, see mk_abi.h); kv_cache [L, 2, smax, hkv, 64] uint16 with positions
     0 .. pos-1 filled; x [d] float32.  `workgroups` must be a multiple of hq (each workgroup takes one
-    (head, context chunk) of the attention) and no more than can be resident at once (one per CU is safe)."""
+    (head, context chunk) of the attention) and no more than can be resident at once: the grid barrier needs every
+    workgroup running, so a count above compute units x the link's workgroups per CU is refused.  After a launch and a
+    synchronize, `raise_on_status(session)` tells whether the step's barriers all completed."""
     smax = kv_cache.shape[2]
     if kv_cache.shape != (layers, 2, smax, hkv, mk.HEAD_DIM) or kv_cache.dtype != np.uint16 or weights.dtype != np.uint16:
         raise ValueError("kv_cache is [L, 2, smax, hkv, 64] uint16, weights uint16")
@@ -36,4 +38,41 @@ def open_session(link_json: str | Path, weights: np.ndarray, kv_cache: np.ndarra
                "h": ((dff,), np.float32), "logits": ((vocab,), np.float32), "sync": ((512,), np.uint32)}
     blob = lambda addr: {"mk.interp": mk.params_blob(addr, num_instr=len(prog), layers=layers, d=d, hq=hq, hkv=hkv, dff=dff,
                                                      vocab=vocab, pos=pos, smax=smax, chunks=chunks)}
-    return open_hostless(link_json, buffers=buffers, params=blob, grid=(workgroups,), backend=backend, image=image)
+    sess = open_hostless(link_json, buffers=buffers, params=blob, grid=(workgroups,), backend=backend, image=image)
+    cus = getattr(sess.backend, "observations", {}).get("observed_cu_count")
+    resident = cus * int(sess.link.get("workgroups_per_cu", 1)) if cus else None
+    if resident is not None and workgroups > resident:
+        sess.close()
+        raise ValueError(f"{workgroups} workgroups cannot all be resident on this device ({resident} at most): the grid barrier would never complete")
+    return sess
+
+
+NUM_XCD = 8
+STATUS_GAVE_UP = 1
+
+
+def raise_on_status(sess: HostlessSession) -> np.ndarray:
+    """Call after `synchronize()`.  Reads the launch's synchronisation words and raises RuntimeError if a barrier wait
+    gave up (status bit 0: the step's outputs are void; x was overwritten, the cache row at `pos` too), if a workgroup
+    has not finished, or if the workgroups that share a per-XCD counter (blockIdx % 8) did not all run on one XCC, or
+    two such groups ran on the same one -- the barrier's first level counts on that.  The status word is cleared, so
+    the session can be launched again.  Returns the words as read."""
+    sync = sess.read("sync")
+    problems = []
+    status = int(sync[1])
+    if status & STATUS_GAVE_UP:
+        problems.append("a grid barrier wait gave up")
+    if status & ~STATUS_GAVE_UP:
+        problems.append(f"unknown status bits {status:#x}")
+    if sync[2] != 0:
+        problems.append(f"{int(sync[2])} workgroups finished without the last one closing the launch")
+    seen = [int(w) for w in sync[288:288 + min(NUM_XCD, sess.grid[0])]]
+    if any(w == 0 or w & (w - 1) for w in seen) or len(set(seen)) != len(seen):
+        problems.append(f"workgroups are not dealt to the XCDs round-robin (XCC bits per blockIdx % 8: {[hex(w) for w in seen]})")
+    if sync[1] != 0:
+        cleared = sync.copy()
+        cleared[1] = 0
+        sess.write("sync", cleared)
+    if problems:
+        raise RuntimeError("decode megakernel: " + "; ".join(problems))
+    return sync

@@ -93,7 +93,8 @@ class MoKSession:
     @staticmethod
     def problem(*, x_q, x_sc, row_token, tokens_per_expert, w_gate_q, w_gate_sc, w_up_q, w_up_sc, w_down_q, w_down_sc,
                 hidden_q, hidden_sc, y, swiglu_limit: float = 7.0) -> MokProblem:
-        """Build the problem record from CUDA tensors (shapes checked here, contents by the library)."""
+        """Build the problem record from CUDA tensors (shapes checked here, contents by the library).  The record
+        keeps references to the tensors (``.tensors``), so it stays valid for as long as the caller holds it."""
         for name, t in dict(x_q=x_q, x_sc=x_sc, tokens_per_expert=tokens_per_expert, w_gate_q=w_gate_q,
                             w_gate_sc=w_gate_sc, w_up_q=w_up_q, w_up_sc=w_up_sc, w_down_q=w_down_q,
                             w_down_sc=w_down_sc, hidden_q=hidden_q, hidden_sc=hidden_sc, y=y).items():
@@ -120,7 +121,7 @@ class MoKSession:
             raise PlkError(3, "weight scales must be slot-major [E, K/128, N, 4] (see weight_scales_to_slot_major)")
         if tokens_per_expert.dtype != torch.int32 or (row_token is not None and row_token.dtype != torch.int32):
             raise PlkError(3, "tokens_per_expert and row_token must be int32")
-        return MokProblem(struct_bytes=sizeof(MokProblem), num_tokens=t_rows, hidden=h, intermediate=i, num_experts=e,
+        prob = MokProblem(struct_bytes=sizeof(MokProblem), num_tokens=t_rows, hidden=h, intermediate=i, num_experts=e,
                           routed_rows=r, ld_sc_h=ldsh, ld_sc_i=ldsi, ld_q_h=ldh, ld_q_i=ldi_q,
                           swiglu_limit=swiglu_limit,
                           x_q=x_q.data_ptr(), x_sc=x_sc.data_ptr(),
@@ -129,6 +130,10 @@ class MoKSession:
                           w_gate_q=w_gate_q.data_ptr(), w_gate_sc=w_gate_sc.data_ptr(), w_up_q=w_up_q.data_ptr(),
                           w_up_sc=w_up_sc.data_ptr(), w_down_q=w_down_q.data_ptr(), w_down_sc=w_down_sc.data_ptr(),
                           hidden_q=hidden_q.data_ptr(), hidden_sc=hidden_sc.data_ptr(), y=y.data_ptr())
+        # the record holds bare addresses: keep the tensors alive as long as it is (a caller may pass temporaries)
+        prob.tensors = (x_q, x_sc, row_token, tokens_per_expert, w_gate_q, w_gate_sc, w_up_q, w_up_sc, w_down_q, w_down_sc,
+                        hidden_q, hidden_sc, y)
+        return prob
 
     def status(self, stream: int | None = None) -> int:
         """Waits for the stream, then returns and clears the launches' sticky status word (``plk_mok_status``): 0, or

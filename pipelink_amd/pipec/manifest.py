@@ -25,7 +25,8 @@ from typing import Any
 from .clauses import ClauseFailure, SchemaError
 from .gfx950 import Profile, get_profile
 
-SCHEMA_VERSIONS = ("3.0",)
+SCHEMA_VERSIONS = ("3.0", "2.0-draft")  # 2.0-draft: the legacy stage schema, which has no tensor section
+TENSOR_SCHEMA_VERSIONS = ("3.0",)
 _STAGE_ID = re.compile(r"[a-z][a-z0-9_-]*(\.[a-z0-9][a-z0-9_-]*)+\Z")
 _HANDLE = re.compile(r"pipelink_[a-z0-9_]+\Z")
 _IDENT = re.compile(r"[A-Za-z_][A-Za-z0-9_]*\Z")
@@ -267,6 +268,12 @@ def load_stage_manifest(obj: Any) -> Stage:
     if not isinstance(topo, dict) or not isinstance(topo.get("persistent"), bool) or \
             not isinstance(topo.get("scheduler"), str):
         c.add("L-TOPO", "$.topology", "topology must give persistent and scheduler")
+    if "tensor" in obj:
+        from .tensors import check_stage_tensor  # (tensors imports this module)
+
+        schema = obj["pipelink_abi"].get("schema", "3.0") if isinstance(obj.get("pipelink_abi"), dict) else None
+        for path, message, detail in check_stage_tensor(obj["tensor"], schema in TENSOR_SCHEMA_VERSIONS):
+            c.add("T-CONTRACT", path, message, **detail)
     c.finish()
     return Stage(obj, profile)  # type: ignore[arg-type]
 

@@ -54,6 +54,84 @@ class TensorPlan:
                 "route": self.route}
 
 
+# What a consumer may promise about the place it calls an import from: a closed vocabulary (the generated function
+# relies on exactly these; docs/reference/tensor-imports.md:96-118 in the reference).
+SITE_GUARANTEES = ("enter_once", "converged", "full_warps", "no_early_return")
+LEND_BINDINGS = ("fixed", "relocatable")
+
+
+def check_stage_tensor(tensor: Any, schema_admits_tensor: bool) -> list[tuple[str, str, dict[str, Any]]]:
+    """Load-time checks of a stage manifest's ``tensor`` section; returns (path, message, detail) per T-CONTRACT
+    failure (the reference's load_stage_tensor, pipec/src/pipec2/tensor/contracts.py, reports the same paths).
+
+    Besides the export and import records the planner reads, a section may carry
+      ``sites``           [{name, role, guarantees: [...]}]: where the stage calls its imports from, and what it
+                          promises there -- tokens of SITE_GUARANTEES only;
+      ``imports[].lends`` [{name, binding, location: {handle, base}, ...}]: resources the consumer lends to the
+                          generated function (scratch memory, a barrier, registers); names are local to the stage
+                          and unique across its imports, and a relocatable lend names the handle the linker places
+                          even when it also states a base.
+    The route table of this linker needs nothing lent, so no stage here declares lends; they are part of the
+    manifest format and are checked where present."""
+    out: list[tuple[str, str, dict[str, Any]]] = []
+    if not schema_admits_tensor:
+        return [("$.tensor", "this stage schema has no tensor section", {})]
+    if not isinstance(tensor, dict):
+        return [("$.tensor", "tensor section must be an object", {})]
+    for kind in ("exports", "imports", "sites"):
+        if not isinstance(tensor.get(kind, []), list):
+            out.append((f"$.tensor.{kind}", f"{kind} must be an array", {}))
+    site_names: set[str] = set()
+    for i, site in enumerate(tensor.get("sites", []) if isinstance(tensor.get("sites", []), list) else []):
+        path = f"$.tensor.sites[{i}]"
+        if not isinstance(site, dict) or not isinstance(site.get("name"), str):
+            out.append((path, "a site is an object with a name", {}))
+            continue
+        if site["name"] in site_names:
+            out.append((f"{path}.name", "site name is declared twice", {"name": site["name"]}))
+        site_names.add(site["name"])
+        promised = site.get("guarantees", [])
+        if not isinstance(promised, list):
+            out.append((f"{path}.guarantees", "guarantees must be an array", {}))
+            continue
+        for j, token in enumerate(promised):
+            if token not in SITE_GUARANTEES:
+                out.append((f"{path}.guarantees[{j}]", "unknown site guarantee", {"allowed": list(SITE_GUARANTEES), "actual": token}))
+            elif token in promised[:j]:
+                out.append((f"{path}.guarantees[{j}]", "site guarantee is listed twice", {"actual": token}))
+    lent: set[str] = set()
+    for i, imp in enumerate(tensor.get("imports", []) if isinstance(tensor.get("imports", []), list) else []):
+        path = f"$.tensor.imports[{i}]"
+        if not isinstance(imp, dict) or not isinstance(imp.get("name"), str):
+            out.append((path, "an import is an object with a name", {}))
+            continue
+        for j, site in enumerate(imp.get("sites", []) or []):
+            if site not in site_names:
+                out.append((f"{path}.sites[{j}]", "import names a site the stage does not declare", {"actual": site}))
+        lends = imp.get("lends", [])
+        if not isinstance(lends, list):
+            out.append((f"{path}.lends", "lends must be an array", {}))
+            continue
+        for j, lend in enumerate(lends):
+            lp = f"{path}.lends[{j}]"
+            if not isinstance(lend, dict) or not isinstance(lend.get("name"), str):
+                out.append((lp, "a lend is an object with a name", {}))
+                continue
+            if lend["name"] in lent:
+                out.append((f"{lp}.name", "two lends publish the same stage-local name", {"name": lend["name"]}))
+            lent.add(lend["name"])
+            if lend.get("binding") not in LEND_BINDINGS:
+                out.append((f"{lp}.binding", "lend binding must be fixed or relocatable", {"actual": lend.get("binding")}))
+            where = lend.get("location")
+            if not isinstance(where, dict) or set(where) != {"handle", "base"}:
+                out.append((f"{lp}.location", "lend location must give handle and base", {}))
+            elif lend.get("binding") == "relocatable" and not isinstance(where["handle"], str):
+                out.append((f"{lp}.location.handle", "a relocatable lend names the handle the linker places", {}))
+            elif where["handle"] is None and where["base"] is None:
+                out.append((f"{lp}.location", "a fixed lend states a handle or a base", {}))
+    return out
+
+
 def _records(stage: Stage, kind: str) -> dict[str, dict[str, Any]]:
     return {r["name"]: r for r in (stage.manifest.get("tensor") or {}).get(kind, [])}
 

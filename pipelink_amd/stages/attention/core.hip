@@ -115,6 +115,7 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[db][r] = 0.0f;
   float row_max = MASKED, row_sum = 0.0f;
+  bool seen = false;  // this lane's query has met a key it may see (decided on unscaled scores: the scale is the caller's)
 
   // the mask package says which stretch of keys the tile's queries may see at all: blocks [first_block, blocks)
   const int keys = pipelink_call_mask_key_count(&view, q0, q0 + FA_Q_TILE - 1);
@@ -216,7 +217,8 @@ extern "C" __device__ void fa_core_role_core(const void* params, unsigned varian
     row_max = new_max;
     // a query that has not seen a key yet (a window mask: the block's keys are all too old for it) has no real maximum
     // to lean on: its exponentials are taken against +huge instead, which makes every one of them 0
-    const float reference = new_max < 0.01f * MASKED ? -MASKED : new_max;
+    seen = seen || block_max > 0.5f * MASKED;
+    const float reference = seen ? new_max : -MASKED;
     float block_sum = 0.0f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)

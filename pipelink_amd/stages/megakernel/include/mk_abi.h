@@ -50,7 +50,9 @@ typedef struct MkInstr {
  * that returns without the call has the interpreter make it. */
 typedef struct MkPending {
   const MkInstr* norm; /* an rmsnorm instruction whose result the op needs, or null */
-  uint32_t barrier;    /* the barrier generation to wait for, 0: none */
+  uint32_t barrier;    /* the barrier generation to wait for (counted over all launches), if `waiting` */
+  uint32_t waiting;    /* non-zero: a barrier is open */
+  uint32_t gave_up;    /* non-zero (in the workgroup's first thread): a wait of this launch was given up; no more waits */
 } MkPending;
 
 typedef struct MkModel {
@@ -64,9 +66,12 @@ typedef struct MkModel {
   float* logits;           /* [V] */
   const float* rope;       /* [2][32]: cos, sin of pos * theta^(-2 i / 64) */
   const MkInstr* program;
-  uint32_t* sync;          /* [0] grid barrier counter (zero at launch; the kernel leaves it zero), [1] status (non-zero: a
-                              wait gave up), [2] count of workgroups that have finished, [32 * (1 + xcd)] arrivals of
-                              one XCD's workgroups; 512 words, all zero at launch and left zero */
+  uint32_t* sync;          /* 512 words, all zero before the first launch.  [0] grid barrier arrivals, [1] status (bit 0: a
+                              wait gave up; sticky, the host clears it), [2] count of workgroups that have finished
+                              (zero between launches), [3] barriers passed by all launches so far, [32 * (1 + xcd)]
+                              arrivals of one XCD's workgroups and [.. + 1] the generation its leader passed on,
+                              [288 + xcd] bits of the XCCs that the workgroups with blockIdx % 8 == xcd ran on.
+                              Counters only grow, from launch to launch. */
   int32_t num_instr, layers, d, hq, hkv, dff, vocab, pos, smax, chunks;
   float eps, attn_scale_log2e;
 } MkModel;

@@ -8,8 +8,9 @@
 // first asks memory for what no workgroup writes (its first rows of weights, its stretch of the cache) and only
 // then calls back (channel inputs_<op>) to wait for the others: the barrier's 2.5 us and the first loads' latency
 // run side by side.  A normalisation instruction is held back in the same way and runs inside that call.
-// The wait is a bounded poll: a workgroup that gives up raises the status word and goes on, it never
-// spins for ever.
+// The wait is a bounded poll: a workgroup that gives up raises the status word and goes on without waiting for any
+// further barrier of the launch, and so does every workgroup that sees the word raised: a launch never spins for
+// ever, and one that cannot complete its barriers ends within a few give-up periods.
 #include <pipelink/stage.hpp>
 #ifndef PIPELINK_EMIT
 #include "mk_device.hpp"
@@ -34,7 +35,12 @@ extern "C" __device__ int pipelink_mk_opcode_rmsnorm_final();
 extern "C" __device__ int pipelink_mk_opcode_lmhead();
 
 namespace mk_interp {
-constexpr uint32_t SPIN_LIMIT = 1u << 22;
+// A wait that is not answered within this many polls is given up.  A barrier takes about 2.5 us, a poll a fraction of a
+// microsecond to a microsecond: 2^16 polls are some tens of milliseconds, thousands of barriers' worth, and short
+// enough that a launch whose workgroups cannot all be resident ends as an error instead of looking like a hang.
+constexpr uint32_t SPIN_LIMIT = 1u << 16;
+constexpr uint32_t STATUS_EVERY = 256;  // a waiting workgroup looks at the status word every so many polls
+constexpr uint32_t STATUS_GAVE_UP = 1u;
 
 // Arrival and release are both in two levels.  An atomic or a load that every XCD must agree on is performed at
 // the memory side, one after the other: 256 of them on one word cost more than the work between two barriers.
@@ -44,8 +50,20 @@ constexpr uint32_t SPIN_LIMIT = 1u << 22;
 // its XCD in a generation number the others poll in their L2.  No cache is written back or invalidated here: what
 // workgroups hand each other across a barrier is stored and loaded at device scope (mk::shared_store / shared_load),
 // and every wave has waited for its stores (the __syncthreads) before its workgroup is counted.
+//
+// Every counter only grows, from launch to launch: barrier number g of a launch is generation base + g, where base
+// (sync[3]) is the number of barriers all earlier launches passed.  So no word is ever put back to zero, and each
+// word is only ever touched at one scope: the per-XCD words at workgroup scope by that XCD's workgroups, the grid's
+// words at device scope.  (Unsigned wrap-around is harmless: targets are compared by difference or for equality.)
+//
+// The round-robin assumption is recorded, not trusted blindly: every workgroup ORs the bit of the XCC it really runs
+// on (hardware register XCC_ID) into sync[288 + blockIdx % 8]; the host checks after a launch that each of these
+// words names one XCC and no two name the same (host/megakernel.py raise_on_status).
 constexpr int NUM_XCD = 8;
 constexpr int XCD_COUNTER = 32;      // sync[32 * (1 + xcd)]: arrivals; [32 * (1 + xcd) + 1]: generation; one 128-byte line per XCD
+constexpr int XCC_SEEN = 32 * 9;     // sync[288 + xcd]: bits of the XCCs its workgroups ran on (device scope, a line of its own)
+// false: the wait was given up -- by this workgroup now (it then raises the status word), or by any workgroup before
+// (the status word is sticky; the host clears it)
 __device__ __forceinline__ bool poll(uint32_t* word, uint32_t target, bool local, const MkModel& m) {
   for (uint32_t spin = 0; spin < SPIN_LIMIT; ++spin) {
     // local: an atomic add of 0 written out as such -- atomics are performed in the L2, whereas a plain
@@ -64,12 +82,15 @@ __device__ __forceinline__ bool poll(uint32_t* word, uint32_t target, bool local
       seen = later;
     }
     if ((int32_t)(seen - target) >= 0) return true;
+    if ((spin & (STATUS_EVERY - 1)) == STATUS_EVERY - 1 &&
+        __hip_atomic_load(m.sync + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+      return false;  // somebody gave up: this barrier will not complete either
     __builtin_amdgcn_s_sleep(1);
   }
-  __hip_atomic_fetch_or(m.sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_fetch_or(m.sync + 1, STATUS_GAVE_UP, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return false;
 }
-// first half of barrier number `generation` (1, 2, ...): this workgroup has finished what comes before it
+// first half of the barrier of generation `generation` (base + 1, base + 2, ...): this workgroup has finished what comes before it
 __device__ __forceinline__ void grid_arrive(const MkModel& m, uint32_t generation) {
   __syncthreads();  // every wave's stores have been issued and acknowledged by the L2
   if (threadIdx.x == 0) {
@@ -80,17 +101,22 @@ __device__ __forceinline__ void grid_arrive(const MkModel& m, uint32_t generatio
       __hip_atomic_fetch_add(m.sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
-// second half: every workgroup has arrived at barrier number `generation`
-__device__ __forceinline__ void grid_wait(const MkModel& m, uint32_t generation) {
-  if (threadIdx.x == 0) {
+// second half: every workgroup has arrived at the barrier of generation pending->barrier.  After a give-up (its own or
+// one it noticed) a workgroup waits for no barrier of the launch any more: the step's results are void by then, and
+// the launch should end quickly.
+__device__ __forceinline__ void grid_wait(const MkModel& m, MkPending* pending) {
+  if (threadIdx.x == 0 && !pending->gave_up) {
+    const uint32_t generation = pending->barrier;
     const uint32_t xcd = blockIdx.x % NUM_XCD, groups = min((uint32_t)NUM_XCD, gridDim.x);
     uint32_t* mine = m.sync + XCD_COUNTER * (1 + xcd);
+    bool ok;
     if (blockIdx.x < NUM_XCD) {  // this XCD's first workgroup listens for the grid
-      poll(m.sync, generation * groups, false, m);
+      ok = poll(m.sync, generation * groups, false, m);
       __hip_atomic_exchange(mine + 1, generation, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     } else {
-      poll(mine + 1, generation, true, m);
+      ok = poll(mine + 1, generation, true, m);
     }
+    if (!ok) pending->gave_up = 1;
   }
   __syncthreads();
 }
@@ -99,9 +125,9 @@ __device__ __forceinline__ void grid_wait(const MkModel& m, uint32_t generation)
 // The ops' way to their inputs: the open barrier, then the normalisation that is due.
 __device__ __forceinline__ void mk_interp_inputs(const void* view, MkPending* pending) {
   const MkModel& m = *static_cast<const MkModel*>(static_cast<const pipelink_host_view*>(view)->residue);
-  if (pending->barrier != 0) {
-    mk_interp::grid_wait(m, pending->barrier);
-    pending->barrier = 0;
+  if (pending->waiting) {
+    mk_interp::grid_wait(m, pending);
+    pending->waiting = 0;
   }
   if (pending->norm != nullptr) {
     pipelink_call_op_rmsnorm(view, pending->norm);
@@ -125,8 +151,16 @@ extern "C" __device__ void mk_interp_role_worker(const void* params, unsigned va
   (void)variant;
   const MkModel& m = *static_cast<const MkModel*>(params);
   const pipelink_host_view view{params, nullptr};
-  uint32_t passed = 0;
-  MkPending pending{nullptr, 0};
+  // generations go on from where the launch before stopped
+  const uint32_t base = __hip_atomic_load(m.sync + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  uint32_t passed = base;
+  MkPending pending{nullptr, 0, 0, 0};
+  if (threadIdx.x == 0) {
+    // XCC_ID is bits 3:0 of hardware register 20: s_getreg_b32 with size 4, offset 0
+    const uint32_t xcc = (uint32_t)__builtin_amdgcn_s_getreg((3 << 11) | 20) & 0xFu;
+    __hip_atomic_fetch_or(m.sync + mk_interp::XCC_SEEN + blockIdx.x % mk_interp::NUM_XCD, 1u << xcc, __ATOMIC_RELAXED,
+                          __HIP_MEMORY_SCOPE_AGENT);
+  }
   for (int i = 0; i < m.num_instr; ++i) {
     const MkInstr* instr = m.program + i;
     const int op = instr->opcode;  // uniform over the grid; the numbers are bound at link time
@@ -148,21 +182,19 @@ extern "C" __device__ void mk_interp_role_worker(const void* params, unsigned va
     if (instr->barrier_after) {
       mk_interp::grid_arrive(m, ++passed);
       pending.barrier = passed;
+      pending.waiting = 1;
     } else {
       __syncthreads();  // the next op of this workgroup reads what this one left in LDS
     }
   }
   mk_interp_inputs(&view, &pending);
-  // The last workgroup to get here puts the barrier counter back to zero for the next launch: by then every
-  // workgroup has left its last barrier.
+  // The last workgroup to get here records where the next launch's generations start: by then every workgroup has
+  // read this launch's base and left its last barrier.  (Every workgroup arrives at every barrier, waited for or
+  // not, so the counters stay in step with the generation even after a give-up.)
   if (threadIdx.x == 0) {
     const uint32_t before = __hip_atomic_fetch_add(m.sync + 2, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
     if (before == gridDim.x - 1) {
-      __hip_atomic_store(m.sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      for (int x = 0; x < mk_interp::NUM_XCD; ++x) {
-        __hip_atomic_store(m.sync + mk_interp::XCD_COUNTER * (1 + x), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(m.sync + mk_interp::XCD_COUNTER * (1 + x) + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+      __hip_atomic_store(m.sync + 3, passed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(m.sync + 2, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     }
   }

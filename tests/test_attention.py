@@ -150,6 +150,41 @@ def test_window_mask_matches_the_oracle_on_every_head(window):
 
 
 @pytest.mark.gpu
+def test_window_mask_with_a_small_softmax_scale():
+    """A caller's scale far below 1 / sqrt(128): queries whose first streamed block holds no key they may see must
+    still give that block zero weight (whether a query has seen a key is decided on unscaled scores)."""
+    from pipelink_amd.host.attention import open_session
+
+    paths = fa_build.images()
+    q, k, v = oa.inputs(1, 4, 2, 640, seed=9)
+    scale = 2.0 ** -10
+    sess = open_session(paths["window_link_json"], _bits(q), _bits(k), _bits(v), window=100, scale=scale)
+    try:
+        sess.write("o", np.full((1, 640, 512), 0x7FC0, dtype=np.uint16))
+        sess.launch()
+        sess.synchronize()
+        o = _from_bits(sess.read("o"))
+    finally:
+        sess.close()
+    for h in range(4):
+        want = oa.attention_head(q[0, h], k[0, h // 2], v[0, h // 2], scale=scale, window=100)
+        got = o[0, :, h * 128:(h + 1) * 128]
+        assert torch.isfinite(got).all()
+        assert (got - want).abs().max().item() <= 1e-2 * want.abs().max().item(), h
+        assert ((got - want).norm() / want.norm()).item() <= 1e-2, h
+
+
+def test_the_host_rejects_a_scale_that_is_not_positive_and_finite():
+    from pipelink_amd.host.attention import open_session
+
+    q = np.zeros((1, 2, 128, 128), dtype=np.uint16)
+    kv = np.zeros((1, 1, 128, 128), dtype=np.uint16)
+    for bad in (0.0, -0.1, float("inf"), float("nan")):
+        with pytest.raises(ValueError, match="scale"):
+            open_session("unused.json", q, kv, kv, scale=bad)
+
+
+@pytest.mark.gpu
 def test_window_mask_at_the_stated_size_on_sampled_heads():
     """B 4, 32 / 8 heads, S 4096 with a window of 1024 keys: tiles start streaming at their first visible block."""
     from pipelink_amd.host.attention import open_session

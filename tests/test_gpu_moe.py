@@ -240,6 +240,19 @@ def test_device_quantiser_is_bit_exact():
         assert not sc.cpu().numpy()[:, 90:].any()   # pad bytes of the 16-byte-pitched scale rows are zero
     q, sc = mxfp8_quantize_device(x.cuda(), pitch=2944)
     assert np.array_equal(q[:, :2880].cpu().numpy(), mxfp8.mx_quantize(x.numpy())[0]) and not q[:, 2880:].any()
+    # NaN and infinities: a NaN keeps its sign and becomes e4m3's NaN code, an infinity saturates, and either puts its
+    # block at the largest scale byte an fp32 exponent field gives (255 - 8)
+    bad = torch.randn(8, 128, generator=g)
+    bad[0, 3] = float("nan")
+    bad[1, 40] = -float("nan")
+    bad.view(torch.int32)[1, 40] |= -0x80000000   # a NaN with its sign bit set, whatever the line above produced
+    bad[2, 5], bad[2, 70] = float("inf"), -float("inf")
+    bad[3, 0], bad[3, 1] = float("nan"), float("inf")
+    for src in (bad, bad.to(torch.bfloat16)):
+        q, sc = mxfp8_quantize_device(src.cuda())
+        oq, osc = mxfp8.mx_quantize(src.float().numpy())
+        assert np.array_equal(q.cpu().numpy(), oq) and np.array_equal(sc.cpu().numpy()[:, :4], osc[:, :4])
+    assert oq[0, 3] & 0x7F == 0x7F and oq[1, 40] & 0x7F == 0x7F and oq[2, 5] == 0x7E and oq[2, 70] == 0xFE and osc[2, 0] == 247
 
 
 def test_weight_layout_conversions_are_pure_permutations():

@@ -160,3 +160,39 @@ def test_swiglu_special_values(c_oracle):
     assert float(gptoss_swiglu(np.float32([100.0]), np.float32([0.0]), None)[0]) == pytest.approx(100.0)
     for g, u in [(0.3, -2.0), (9.0, 9.0), (-3.0, 0.1)]:
         assert c_oracle.plko_swiglu(g, u, L, 1) == pytest.approx(f(g, u), rel=1e-6, abs=1e-7)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_host_quantiser_equals_the_oracle_bit_for_bit(dtype):
+    """pipelink_amd.mxfp8.quantize (torch; what the harness-side code calls where the reference calls ops.mxfp8_quantize,
+    campaigns/mok/host/mok_port_host.py:122) against oracle.mxfp8.mx_quantize: codes and scale bytes, on random data
+    over 60 binades, blocks of zeros, blocks whose scale sits at 2^+-30, values that saturate after scaling only by
+    rounding, subnormal inputs, NaN of both signs and infinities."""
+    import torch
+    from pipelink_amd import mxfp8 as host
+
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(64, 256, generator=g) * torch.exp2(torch.randint(-30, 31, (64, 8), generator=g).float()).repeat_interleave(32, dim=1)
+    x[0] = 0                                   # a row of zero blocks: scale byte 0, codes 0
+    x[1, :32] = 0
+    x[2, :32] = torch.randn(32, generator=g) * 2.0 ** 30
+    x[3, :32] = torch.randn(32, generator=g) * 2.0 ** -30
+    x[4, :32] = 2.0 ** -130                    # fp32 subnormals: exponent field 0, scale byte 0
+    x[5, 0], x[5, 1:32] = 1.99999, 0.001       # amax just below a power of two: the largest quotient rounds up to 256
+    x[6, 0], x[6, 1] = 255.99, 447.9           # near the top of the e4m3 range before scaling
+    x[7, 3] = float("nan")
+    x[8, 40] = float("nan")
+    x.view(torch.int32)[8, 40] |= -0x80000000  # NaN with the sign bit set
+    x[9, 5], x[9, 70] = float("inf"), -float("inf")
+    src = x.to(getattr(torch, dtype))
+    q, sc = host.quantize(src)
+    oq, osc = mxfp8.mx_quantize(src.float().numpy())
+    assert np.array_equal(q.numpy(), oq)
+    assert np.array_equal(sc.numpy()[:, :8], osc[:, :8]) and not sc.numpy()[:, 8:].any()
+    assert not oq[0].any() and not osc[0].any() and oq[7, 3] & 0x7F == 0x7F and oq[8, 40] & 0x7F == 0x7F and oq[9, 5] == 0x7E and oq[9, 70] == 0xFE
+    if dtype == "float32":  # (torch's conversion to bf16 does not keep a NaN's sign)
+        assert oq[7, 3] == 0x7F and oq[8, 40] == 0xFF
+    # and the inverse maps agree on everything finite
+    back, oback = host.dequantize(q, sc).numpy(), mxfp8.mx_dequantize(oq, osc)
+    fin = np.isfinite(oback)
+    assert np.array_equal(back[fin], oback[fin]) and np.array_equal(np.isnan(back), np.isnan(oback))

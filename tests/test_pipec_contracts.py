@@ -109,8 +109,28 @@ def schema_base():
     return {"stages": [stage("schema.stage", {"load": 4}, variants=variants)]}
 
 
+def tensor_base():
+    """A consumer stage with one tensor import as this linker records it (name, identity, wanted layout, function), the
+    site it calls the import from, and three lends of the kinds the reference's corpus uses (test_tensor_contracts.py:68-80:
+    relocatable scratch memory, a fixed barrier, fixed registers)."""
+    st = stage("tensor.stage", {"epilogue": 4})
+    life = {"from": "tile_ready", "to": "import_complete"}
+    st["tensor"] = {
+        "schema": "tensor-v1", "exports": [],
+        "imports": [{"name": "epilogue", "result": "C", "dtype": "fp32", "shape": [128, 32], "layout": "mfma32x32c",
+                     "fn": "pipelink_import_accumulator", "sites": ["epilogue_hook"],
+                     "lends": [{"name": "scratch", "domain": "smem", "extent": 4096, "align": 128, "scope": "cta", "binding": "relocatable",
+                                "location": {"handle": "pipelink_import_scratch", "base": None}, "owner": "epilogue", "lifetime": life},
+                               {"name": "rendezvous", "domain": "barrier", "extent": 1, "align": 1, "scope": "cta", "binding": "fixed",
+                                "location": {"handle": None, "base": 1}, "owner": "epilogue", "lifetime": life},
+                               {"name": "fragment", "domain": "reg", "extent": 32, "align": 1, "scope": "thread", "binding": "fixed",
+                                "location": {"handle": "private_fragment", "base": None}, "owner": "epilogue", "lifetime": life}]}],
+        "sites": [{"name": "epilogue_hook", "role": "epilogue", "guarantees": ["converged"]}]}
+    return {"stages": [st]}
+
+
 BASES = {"barrier": barrier_base, "double_barrier": double_barrier_base, "call": call_base, "topology": topology_base,
-         "schema": schema_base}
+         "schema": schema_base, "tensor": tensor_base}
 
 
 def set_path(root, path, value):
