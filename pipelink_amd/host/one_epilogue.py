@@ -1,6 +1,6 @@
 """Host side of the one-epilogue-many-producers example (C = (A . B) * scale[col] + bias[col]) on the
-host-less route: the same buffers and params for each of the three linked pipelines (accumulator in
-AGPRs, VGPRs, LDS) and their one-unit controls."""
+host-less route: the same buffers and params for each of the linked pipelines (accumulator in AGPRs,
+VGPRs, LDS with 128 x 128 workgroup tiles; `wide`: 256 x 128 tiles, accumulator in AGPRs) and their one-unit controls."""
 from __future__ import annotations
 
 from pathlib import Path
@@ -22,9 +22,10 @@ def open_session(link_json: str | Path, home: str, a_bits: np.ndarray, bt_bits: 
     n, k2 = bt_bits.shape
     if k != k2 or bias.shape != (n,) or scale.shape != (n,):
         raise ValueError("operand shapes do not agree")
-    if m % TILE or n % TILE or k % TILE_K or a_bits.dtype != np.uint16 or bt_bits.dtype != np.uint16:
-        raise ValueError("m and n must be multiples of 128, k of 64, operands uint16 bf16 bit patterns")
+    tile_m, tile_n = (256, 128) if home == "wide" else (TILE, TILE)
+    if m % tile_m or n % tile_n or k % TILE_K or a_bits.dtype != np.uint16 or bt_bits.dtype != np.uint16:
+        raise ValueError(f"m must be a multiple of {tile_m}, n of {tile_n}, k of 64, operands uint16 bf16 bit patterns")
     buffers = {"a": a_bits, "bt": bt_bits, "bias": bias.astype(np.float32), "scale": scale.astype(np.float32),
                "c": ((m, n), np.uint16), "status": ((1,), np.uint32)}
     return open_hostless(link_json, buffers=buffers, params=lambda addr: params_blobs(addr, m, n, k, home),
-                         grid=((m // TILE) * (n // TILE),), backend=backend, image=image)
+                         grid=((m // tile_m) * (n // tile_n),), backend=backend, image=image)

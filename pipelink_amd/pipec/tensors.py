@@ -5,8 +5,8 @@ per-participant shape) and its placement -- the *home* (``agpr``, ``vgpr`` or ``
 that home.  A consumer package imports one (``PL_IMPORT_TENSOR``): the same identity, the layout it wants
 the elements in, and the name of a function it calls to get them.  The pipeline connects an export to an
 import (``tensor_connections``); the linker checks the identities (``T-CONTRACT``), picks a route
-(``T-PLAN`` if none exists) and *generates* the function, together with ``<fn>_ready()`` and
-``<fn>_done()``, into the binding stubs.  The consumer's source never changes with the producer's home.
+(``T-PLAN`` if none exists) and *generates* the function, together with ``<fn>_ready()``,
+``<fn>_done()`` and ``<fn>_block()`` (one 32 x 32 block at a time), into the binding stubs.  The consumer's source never changes with the producer's home.
 
 The reference plans such routes with a model of typed transport primitives and a bounded search
 (pipec/src/pipec2/tensor/plan.py:557 ``ConnectionPlanner``, lowering in tensor/lower.py:679; contract in
@@ -223,5 +223,22 @@ def generate_adapters(plans: list[TensorPlan]) -> str:
                     "        const int row = 32 * i + 8 * (r / 4) + 4 * (lane >> 5) + r % 4, col = 32 * j + (lane & 31);",
                     f"        dest[(i * {bj} + j) * 16 + r] = *reinterpret_cast<const float*>(tile + row * {pitch} + col * 4);",
                     "      }"]
+        out += ["}"]
+        # the same, one 32 x 32 block (16 elements per lane, block = i * (cols / 32) + j) at a time: for a consumer whose
+        # registers do not hold the whole tensor
+        out.append(f'extern "C" __device__ __attribute__((always_inline)) void {fn}_block(const void* source, int block, float* dest) {{')
+        if p.route == "register_copy":
+            out += ["  const float* frame = static_cast<const float*>(source) + block * 16;", "#pragma unroll",
+                    "  for (int k = 0; k < 16; ++k) dest[k] = frame[k];"]
+        elif p.route == "accvgpr_receipt":
+            out += ["  const float* frame = static_cast<const float*>(source) + block * 16;", "#pragma unroll",
+                    "  for (int k = 0; k < 16; ++k) {", "    float v;",
+                    '    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(frame[k]));', "    dest[k] = v;", "  }"]
+        else:
+            out += ["  const unsigned char* tile = static_cast<const unsigned char*>(source);",
+                    f"  const int lane = threadIdx.x & 63, i = block / {bj}, j = block % {bj};", "#pragma unroll",
+                    "  for (int r = 0; r < 16; ++r) {",
+                    "    const int row = 32 * i + 8 * (r / 4) + 4 * (lane >> 5) + r % 4, col = 32 * j + (lane & 31);",
+                    f"    dest[r] = *reinterpret_cast<const float*>(tile + row * {pitch} + col * 4);", "  }"]
         out += ["}", ""]
     return "\n".join(out)

@@ -2,9 +2,11 @@
 three-package GEMM example, unchanged), three matrix packages that keep their accumulator in AGPRs, in
 VGPRs and in an LDS tile, and ONE epilogue package; links the epilogue against each producer in turn
 (the linker generates the accumulator import for each home) and builds each pipeline's one-unit control.
+A fourth pipeline, ``wide``, is the same composition at the tile size the accumulation registers allow
+(256 x 128 per workgroup, 128 x 64 per wave): its own loader, matrix and epilogue packages.
 
 Counterpart of examples/one-epilogue-many-producers/build.py in the reference.  Output under
-``build/``: the five ``.plink`` packages and, per home, ``<home>/{pipeline.json, link/..., one_unit.hsaco}``."""
+``build/``: the ``.plink`` packages and, per home (and ``wide``), ``<home>/{pipeline.json, link/..., one_unit.hsaco}``."""
 from __future__ import annotations
 
 import json
@@ -15,8 +17,15 @@ from pathlib import Path
 HERE = Path(__file__).resolve().parent
 BUILD = HERE / "build"
 HOMES = ("agpr", "vgpr", "lds")
+WIDE = "wide"   # the 256 x 128 tile: its own loader, matrix and epilogue packages (accumulator in 128 AGPRs)
 PACKAGES = [("gs.loader", HERE.parent / "gemm_split" / "loader.hip"), ("oe.mma.agpr", HERE / "mma_agpr.hip"),
-            ("oe.mma.vgpr", HERE / "mma_vgpr.hip"), ("oe.mma.lds", HERE / "mma_lds.hip"), ("oe.epilogue", HERE / "epilogue.hip")]
+            ("oe.mma.vgpr", HERE / "mma_vgpr.hip"), ("oe.mma.lds", HERE / "mma_lds.hip"), ("oe.epilogue", HERE / "epilogue.hip"),
+            ("oe.loader.wide", HERE / "loader_wide.hip"), ("oe.mma.wide", HERE / "mma_wide.hip"),
+            ("oe.epilogue.wide", HERE / "epilogue_wide.hip")]
+
+
+def _stages_of(cell_name: str) -> tuple[str, ...]:
+    return ("oe.loader.wide", "oe.mma.wide", "oe.epilogue.wide") if cell_name == WIDE else ("gs.loader", f"oe.mma.{cell_name}", "oe.epilogue")
 
 
 def build(out: Path = BUILD, one_unit: bool = True) -> dict:
@@ -25,10 +34,10 @@ def build(out: Path = BUILD, one_unit: bool = True) -> dict:
     out.mkdir(parents=True, exist_ok=True)
     reports = {sid: pack.pack_stage(src, out / f"{sid}.plink") for sid, src in PACKAGES}
     links, controls = {}, {}
-    for home in HOMES:
+    for home in HOMES + (WIDE,):
         cell = out / home
         cell.mkdir(exist_ok=True)
-        for sid in ("gs.loader", f"oe.mma.{home}", "oe.epilogue"):
+        for sid in _stages_of(home):
             shutil.copy(out / f"{sid}.plink", cell / f"{sid}.plink")
         shutil.copy(HERE / f"pipeline_{home}.json", cell / "pipeline.json")
         links[home] = linker.link(cell / "pipeline.json", cell / "link")

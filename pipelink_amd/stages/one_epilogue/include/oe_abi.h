@@ -18,6 +18,11 @@
 #define OE_STAGE_BYTES (2 * 128 * 128)
 #define OE_LOAD_WAVES 2 /* the loader's waves: arrivals on a stage's `full` counter per fill (GS_LOAD_WAVES) */
 #define OE_LDS_PITCH (64 * 4 + 16) /* bytes between rows of a wave's 64 x 64 fp32 tile in LDS */
+/* the wide trio (oe.loader.wide, oe.mma.wide, oe.epilogue.wide): a 256 x 128 workgroup tile, a wave's share 128 x 64 */
+#define OE_WIDE_TILE_M 256
+#define OE_WIDE_TILE_N 128
+#define OE_WIDE_STAGE_BYTES ((256 + 128) * 128) /* 64 contraction elements of 256 A rows, then of 128 B^T rows */
+#define OE_WIDE_LOAD_WAVES 3                    /* 128 rows each: upper A, lower A, B^T */
 
 typedef struct OeMmaParams {
   uint32_t* status;
@@ -32,7 +37,16 @@ typedef struct OeEpilogueParams {
 } OeEpilogueParams;
 
 typedef struct OeTile {
-  int32_t row0, col0; /* first row / column of the calling wave's 64 x 64 share */
+  int32_t row0, col0; /* first row / column of the calling wave's share (64 x 64; 128 x 64 in the wide trio) */
 } OeTile;
+
+/* the wide loader's params: the layout of the three-package example's GsLoaderParams */
+typedef struct OeLoaderParams {
+  const uint16_t* a;  /* [M, K] bf16 */
+  const uint16_t* bt; /* [N, K] bf16 */
+  uint32_t* status;   /* [1], set to non-zero by a wait that gave up */
+  int32_t m, n, k;    /* multiples of 256, 128, 64 */
+  int32_t reserved;
+} OeLoaderParams;
 
 #endif

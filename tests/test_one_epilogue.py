@@ -79,6 +79,24 @@ def _relink(example_dir: Path, tmp_path: Path, home: str, stage_id: str | None, 
 
 
 @needs_rocm
+def test_wide_tile_links_its_own_trio(example):
+    """256 x 128 workgroup tiles: three loader waves + four matrix waves, three stages of 48 KB in the ring, the wave's
+    128 x 64 accumulator in AGPRs handed to the epilogue one 32 x 32 block at a time."""
+    out, res = example
+    wide = res["links"]["wide"]
+    assert [e["stage_id"] for e in wide["params"]["entries"]] == ["oe.loader.wide", "oe.mma.wide", "oe.epilogue.wide"]
+    assert wide["threads"] == 7 * 64 and wide["bindings"]["pipelink_gs_depth"] == [3, "solved"]
+    assert wide["dyn_smem_bytes"] == 3 * (256 + 128) * 128 + 2 * 3 * 16 <= 160 * 1024
+    plan = wide["tensor_plans"][0]
+    assert plan["route"] == "accvgpr_receipt" and plan["function"] == "oe_epilogue_wide_import_acc"
+    obs = wide["observed"]
+    # two waves share a SIMD (7 waves on 4): 256 registers each at most
+    assert obs["calls"] == 0 and obs["private_segment_fixed_size"] == 0 and obs["agpr_count"] == 128 and obs["vgpr_count"] <= 256
+    stub = (out / "wide" / "link" / "stub.hip").read_text()
+    assert "oe_epilogue_wide_import_acc_block(const void* source, int block, float* dest)" in stub
+
+
+@needs_rocm
 def test_rejected_tensor_connections_are_named(example, tmp_path):
     cases = [
         ("vgpr", "oe.mma.vgpr", lambda m: m["tensor"]["exports"][0].update(dtype="f16"), None, "T-CONTRACT",
@@ -115,7 +133,7 @@ def test_three_homes_one_epilogue_bit_exact_and_within_the_bf16_bar(size):
     a, b, scale, bias = gg.scale_bias_inputs(size, size, size, seed=0)
     a_bits, bt_bits = _bits(a), _bits(b.t())
     results = {}
-    for home in oe_build.HOMES:
+    for home in oe_build.HOMES + (oe_build.WIDE,):
         paths = oe_build.images(home)
         sess = open_session(paths["link_json"], home, a_bits, bt_bits, bias.numpy(), scale.numpy())
         try:
@@ -133,6 +151,8 @@ def test_three_homes_one_epilogue_bit_exact_and_within_the_bf16_bar(size):
         finally:
             sess.close()
     assert np.array_equal(results["agpr"], results["vgpr"]) and np.array_equal(results["agpr"], results["lds"])
+    # the wide tile multiplies the same 16-element steps in the same order: the same bits
+    assert np.array_equal(results["agpr"], results["wide"])
     rows = torch.arange(size) if size <= 512 else torch.from_numpy(np.random.default_rng(0).choice(size, 48, replace=False))
     want = gg.gemm_scale_bias_torch(a, b, scale, bias, rows).float().numpy()
     got = torch.from_numpy(results["agpr"].view(np.int16)).view(torch.bfloat16).float().numpy()[rows.numpy()]
