@@ -134,6 +134,24 @@ def test_tiles_at_the_end_of_an_experts_rows(cell):
         assert moe_ffn.rel_frobenius(mxfp8.mx_dequantize(hq, hsc), mxfp8.mx_dequantize(ref["hidden_q"], ref["hidden_sc"])) <= TOL
 
 
+def test_down_tiles_wait_for_rows_another_xcd_produces(cell):
+    """One launch, shaped so that the dependency wait is really taken: two experts of 17 and 7 row tiles, ONE gate/up
+    column tile and four down column tiles.  An XCD's list holds 3 gate/up tiles and then 12 down tiles, whose rows are
+    almost all produced by gate/up tiles on other XCDs' lists: the first down tile of most workgroups has to wait for a
+    readiness counter another XCD bumps.  Must equal the two launches byte for byte, with no give-up."""
+    from pipelink_amd.host import mok_inputs
+
+    T, H, I = 1024, 1024, 128
+    inp = mok_inputs.generate(T, H, I, 2, 1, seed=57, counts=[16 * 256 + 17, 6 * 256 + 200])
+    two = _run(cell[0], inp, H, I, pitch_i=I + 16)      # a pitch that is not a multiple of 128: two launches
+    ref = _oracle(inp)
+    assert moe_ffn.rel_frobenius(two[2].float().numpy(), ref["y"]) <= TOL
+    for _ in range(3):                                   # the race, if there were one, need not show the first time
+        one = _run(cell[0], inp, H, I, pitch_i=I)
+        assert np.array_equal(one[0], two[0]) and np.array_equal(one[1][:, :I // 32], two[1][:, :I // 32])
+        assert torch.equal(one[2].view(torch.int16), two[2].view(torch.int16))
+
+
 def test_one_launch_forward_twice_on_the_same_buffers(cell):
     """Two forwards in a row that share hidden / y buffers but not inputs: the second must not read anything of the
     first (its `hidden` rows as an XCD's cache may still hold them) -- against a forward into fresh buffers; and a
