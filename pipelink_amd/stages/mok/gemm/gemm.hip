@@ -336,7 +336,12 @@ __device__ __forceinline__ void wait_rows(const MokGemmTask& t, const MokCounter
   if (!waits(t, counters)) return;
   if (threadIdx.x == 0) {
     bool ok = false;
-    for (uint32_t spin = 0; spin < WAIT_POLLS; ++spin) {
+    uint32_t limit = WAIT_POLLS;
+    if (counters.status) {  // the host may shorten the wait (MOK_WS_POLL_LIMIT)
+      const uint32_t asked = __hip_atomic_load(counters.status + (MOK_WS_POLL_LIMIT - MOK_WS_STATUS), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (asked != 0) limit = asked;
+    }
+    for (uint32_t spin = 0; spin < limit; ++spin) {
       if (__hip_atomic_load(counters.base + t.counter_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= t.wait_target) {
         ok = true;
         break;

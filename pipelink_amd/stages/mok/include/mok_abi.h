@@ -112,6 +112,8 @@ typedef struct MokFrameworkParams {
 enum {
   MOK_WS_STATUS = 0,    /* sticky MOK_STATUS_* bits; the host reads and clears it */
   MOK_WS_FINISHED = 1,  /* workgroups that have left the launch; the last one clears the counters */
+  MOK_WS_POLL_LIMIT = 2, /* 0, or the number of polls after which a dependency wait gives up instead of the default 2^18
+                            (for tests of the give-up path: the kernels never write it) */
   MOK_WS_COUNTERS = 32  /* first readiness counter */
 };
 

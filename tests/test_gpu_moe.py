@@ -340,6 +340,61 @@ def test_broker_route_gives_the_same_bytes_as_the_forward_entry(cell):
         assert not t["workspace"].cpu().any()   # the launch left its counters at zero and raised no status bit
 
 
+def test_a_dependency_wait_that_cannot_be_met_gives_up_and_says_so(cell):
+    """The bounded wait, forced from the host: the readiness counters start far below zero, so no row tile ever reads
+    complete, and the poll limit (workspace word 2) is set to a handful.  The launch must end, raise status bit 0 and leave
+    its counters at zero; the next launch on a clean workspace is correct again."""
+    import json
+    from pipelink_amd.host import broker, mok_inputs
+    from pipelink_amd.host.backend import HipBackend
+    from pipelink_amd.host.mok import scale_pitch, weight_codes_to_k64_tiled, weight_scales_to_slot_major
+    from pipelink_amd.stages.mok import build as mok_build
+
+    T, H, I, E, k, PITCH = 300, 320, 192, 4, 2, 256
+    inp = mok_inputs.generate(T, H, I, E, k, seed=1)
+    want = _run(cell[0], inp, H, I, pitch_i=PITCH)
+    dev = torch.device("cuda:0")
+    d = {n: v.to(dev) for n, v in inp.__dict__.items()}
+    t = dict(x_q=d["x_q"], x_sc=d["x_sc"], row_token=d["row_token"], tokens_per_expert=d["tokens_per_expert"],
+             w_gate_q=weight_codes_to_k64_tiled(d["w_gate_q"], H), w_gate_sc=weight_scales_to_slot_major(d["w_gate_sc"], H),
+             w_up_q=weight_codes_to_k64_tiled(d["w_up_q"], H), w_up_sc=weight_scales_to_slot_major(d["w_up_sc"], H),
+             w_down_q=weight_codes_to_k64_tiled(d["w_down_q"], I), w_down_sc=weight_scales_to_slot_major(d["w_down_sc"], I))
+    rows = int(inp.tokens_per_expert.sum())
+    words = 32 + (rows + 255) // 256 + E
+    t["hidden_q"] = torch.full((rows, PITCH), 0xFF, dtype=torch.uint8, device=dev)
+    t["hidden_sc"] = torch.full((rows, scale_pitch(I)), 0xFF, dtype=torch.uint8, device=dev)
+    t["y"] = torch.full((rows, H), float("nan"), dtype=torch.bfloat16, device=dev)
+    ws = torch.zeros(words, dtype=torch.int32)
+    tiles = int(((inp.tokens_per_expert + 255) // 256).sum())   # the row tiles there are (the workspace has room for more)
+    ws[2] = 4                 # give up after four polls
+    ws[32:32 + tiles] = -1000  # no counter can reach its target
+    t["workspace"] = ws.to(dev)
+    res = lambda n: broker.Resource(t[n].data_ptr(), t[n].numel() * t[n].element_size())
+    resources = {"mok.framework": {"tokens_per_expert": res("tokens_per_expert"), "workspace": res("workspace")},
+                 "mok.gemm": {n: res(n) for n in ("x_q", "x_sc", "w_gate_q", "w_gate_sc", "w_up_q", "w_up_sc", "w_down_q",
+                                                  "w_down_sc", "hidden_q", "hidden_sc", "y", "row_token")},
+                 "mok.act": {"hidden_q": res("hidden_q"), "hidden_sc": res("hidden_sc")}}
+    scalars = {"mok.num_local_tokens": T, "mok.hidden": H, "mok.intermediate": I, "mok.num_local_experts": E,
+               "mok.swiglu_limit": 7.0, "mok.pass": 0, "mok.precision": 1, "mok.routed_rows": rows, "mok.ld_q_h": H,
+               "mok.ld_q_i": PITCH, "mok.ld_sc_h": scale_pitch(H), "mok.ld_sc_i": scale_pitch(I), "mok.workspace_words": words}
+    paths = mok_build.images()
+    link = json.loads(paths["link_json"].read_text())
+    be = HipBackend(0, torch.cuda.current_stream().cuda_stream)
+    with broker.open_host(link, paths["linked"].read_bytes(), resources, scalars, be) as s:
+        s.launch()
+        be.synchronize()
+        after = t["workspace"].cpu()
+        assert after[0] == 1                                   # MOK_STATUS_WAIT_GAVE_UP
+        assert after[1] == 0 and not after[32:].any()          # the launch closed and put its counters back
+        assert np.array_equal(t["hidden_q"][:, :I].cpu().numpy(), want[0])   # the gate/up tiles depend on nobody
+        t["workspace"].zero_()                                 # the host clears the status (and the poll limit)
+        t["y"].fill_(float("nan"))
+        s.launch()
+        be.synchronize()
+        assert not t["workspace"].cpu().any()
+        assert torch.equal(t["y"].cpu().view(torch.int16), want[2].view(torch.int16))
+
+
 def test_launch_verb_runs_both_passes_through_the_providers(cell, tmp_path):
     """`pipec launch LINK --provider GROUP=SO ... --host-inputs JSON` (cli.py:226-258 in the reference): buffers from
     files, one launch per invocation, outputs written back to files -- against the forward entry's bytes."""
