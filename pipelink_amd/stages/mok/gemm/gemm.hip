@@ -367,8 +367,8 @@ __device__ __forceinline__ Views views_of(const MokGemmResidue& g, const MokGemm
 }
 
 // The gathered part of a tile's loader: routed row -> source row goes through row_token for the gate/up op, a
-// dependent load: from LDS if the task was staged (tokens of rows past the end are zero there), else from memory.
-__device__ __forceinline__ void gather_rows(const MokGemmResidue& g, const Views& v, const MokGemmTask& t, GemmCarry& c, bool staged) {
+// dependent load, which `stage` has taken ahead: the tokens are read from LDS (those of rows past the end are zero there).
+__device__ __forceinline__ void gather_rows(const MokGemmResidue& g, const Views& v, const MokGemmTask& t, GemmCarry& c) {
   const int tid = fresh_tid();
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -383,13 +383,13 @@ __device__ __forceinline__ void gather_rows(const MokGemmResidue& g, const Views
     const int trow = (wave * X_GROUPS + i) * 16 + lrow;  // tile-local routed row
     const int row = t.row_begin + trow;
     const int safe = row < t.row_end ? row : t.row_end - 1;
-    const int src = !gathered ? safe : staged ? staged_token[trow] : g.row_token[safe];
+    const int src = gathered ? staged_token[trow] : safe;
     c.xsrc[i] = row < t.row_end ? (uint32_t)src * (uint32_t)act.ld_q + chunk : PAST_THE_END;
   }
   // routed-row scales: thread tid fetches row tid's 16-byte piece
   const int row = t.row_begin + tid;
   const int safe = row < t.row_end ? row : t.row_end - 1;
-  const int src = !gathered ? safe : staged ? staged_token[tid] : g.row_token[safe];
+  const int src = gathered ? staged_token[tid] : safe;
   c.xscsrc = row < t.row_end ? (uint32_t)src * (uint32_t)act.ld_sc : PAST_THE_END;
 }
 
@@ -483,9 +483,9 @@ __device__ __forceinline__ int loads_younger_than_slot(int slot, int last, int n
 }
 
 template <int DEPTH>
-__device__ __forceinline__ void prefetch(const MokGemmResidue& g, const MokGemmTask& t, GemmCarry& c, bool staged) {
+__device__ __forceinline__ void prefetch(const MokGemmResidue& g, const MokGemmTask& t, GemmCarry& c) {
   const Views v = views_of(g, t);
-  gather_rows(g, v, t, c, staged);
+  gather_rows(g, v, t, c);
   const Loader ld = make_loader(v, t, c);
   const Rings<DEPTH> r;
   const int n = v.act.k / K_SLOT;
@@ -823,8 +823,8 @@ extern "C" __device__ void mok_gemm_wait(const void* view, const MokGemmTask* ta
 extern "C" __device__ void mok_gemm_prefetch(const void* view, const MokGemmTask* task, mok::GemmCarry* carry) {
   const auto& g = mok_gemm_residue(view);
   switch (pipelink_mok_gemm_depth()) {  // a link-time constant: one case survives
-    case 2: mok_gemm_owner::prefetch<2>(g, *task, *carry, true); break;
-    default: mok_gemm_owner::prefetch<4>(g, *task, *carry, true); break;
+    case 2: mok_gemm_owner::prefetch<2>(g, *task, *carry); break;
+    default: mok_gemm_owner::prefetch<4>(g, *task, *carry); break;
   }
 }
 
