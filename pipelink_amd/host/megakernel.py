@@ -35,7 +35,7 @@ def open_session(link_json: str | Path, weights: np.ndarray, kv_cache: np.ndarra
     prog = mk.program(layers, mk.opcodes_of(link))   # the instruction stream speaks the numbers this link bound
     buffers = {"weights": weights, "kv_cache": kv_cache, "x": x.astype(np.float32), "rope": mk.rope_table(pos), "program": prog,
                "qkv": (((hq + 2 * hkv) * mk.HEAD_DIM,), np.float32), "attn_partial": ((hq * chunks * mk.PARTIAL_STRIDE,), np.float32),
-               "h": ((dff,), np.float32), "logits": ((vocab,), np.float32), "sync": ((512,), np.uint32)}
+               "h": ((dff,), np.float32), "logits": ((vocab,), np.float32), "sync": ((1024,), np.uint32)}
     blob = lambda addr: {"mk.interp": mk.params_blob(addr, num_instr=len(prog), layers=layers, d=d, hq=hq, hkv=hkv, dff=dff,
                                                      vocab=vocab, pos=pos, smax=smax, chunks=chunks)}
     sess = open_hostless(link_json, buffers=buffers, params=blob, grid=(workgroups,), backend=backend, image=image)
@@ -55,7 +55,7 @@ def raise_on_status(sess: HostlessSession) -> np.ndarray:
     """Call after `synchronize()`.  Reads the launch's synchronisation words and raises RuntimeError if a barrier wait
     gave up (status bit 0: the step's outputs are void; x was overwritten, the cache row at `pos` too), if a workgroup
     has not finished, or if the workgroups that share a per-XCD counter (blockIdx % 8) did not all run on one XCC, or
-    two such groups ran on the same one -- the barrier's first level counts on that.  The status word is cleared, so
+    two such groups ran on the same one (as recorded by the session's first launch) -- the barrier's first level counts on that.  The status word is cleared, so
     the session can be launched again.  Returns the words as read."""
     sync = sess.read("sync")
     problems = []
@@ -66,9 +66,11 @@ def raise_on_status(sess: HostlessSession) -> np.ndarray:
         problems.append(f"unknown status bits {status:#x}")
     if sync[2] != 0:
         problems.append(f"{int(sync[2])} workgroups finished without the last one closing the launch")
-    seen = [int(w) for w in sync[288:288 + min(NUM_XCD, sess.grid[0])]]
-    if any(w == 0 or w & (w - 1) for w in seen) or len(set(seen)) != len(seen):
-        problems.append(f"workgroups are not dealt to the XCDs round-robin (XCC bits per blockIdx % 8: {[hex(w) for w in seen]})")
+    if sync[3] != 0:  # at least one launch has closed: its workgroups recorded where they ran
+        ran_on = sync[512:512 + min(512, sess.grid[0])]
+        groups = [sorted({int(w) for w in ran_on[x::NUM_XCD]}) for x in range(min(NUM_XCD, sess.grid[0]))]
+        if any(len(g) != 1 or not g[0] & 0x100 for g in groups) or len({g[0] for g in groups}) != len(groups):
+            problems.append(f"workgroups are not dealt to the XCDs round-robin (recorded XCC words per blockIdx % 8: {groups})")
     if sync[1] != 0:
         cleared = sync.copy()
         cleared[1] = 0

@@ -50,9 +50,7 @@ typedef struct MkInstr {
  * that returns without the call has the interpreter make it. */
 typedef struct MkPending {
   const MkInstr* norm; /* an rmsnorm instruction whose result the op needs, or null */
-  uint32_t barrier;    /* the barrier generation to wait for (counted over all launches), if `waiting` */
-  uint32_t waiting;    /* non-zero: a barrier is open */
-  uint32_t gave_up;    /* non-zero (in the workgroup's first thread): a wait of this launch was given up; no more waits */
+  uint32_t barrier;    /* the barrier of this launch to wait for (1, 2, ...), 0: none */
 } MkPending;
 
 typedef struct MkModel {
@@ -66,12 +64,12 @@ typedef struct MkModel {
   float* logits;           /* [V] */
   const float* rope;       /* [2][32]: cos, sin of pos * theta^(-2 i / 64) */
   const MkInstr* program;
-  uint32_t* sync;          /* 512 words, all zero before the first launch.  [0] grid barrier arrivals, [1] status (bit 0: a
-                              wait gave up; sticky, the host clears it), [2] count of workgroups that have finished
-                              (zero between launches), [3] barriers passed by all launches so far, [32 * (1 + xcd)]
-                              arrivals of one XCD's workgroups and [.. + 1] the generation its leader passed on,
-                              [288 + xcd] bits of the XCCs that the workgroups with blockIdx % 8 == xcd ran on.
-                              Counters only grow, from launch to launch. */
+  uint32_t* sync;          /* 1024 words, all zero before the first launch.  [0] grid barrier arrivals, [1] status (bit 0: a
+                              wait gave up; sticky, the host clears it), [2] count of workgroups that have finished,
+                              [3] launches closed so far, [32 * (1 + xcd)] arrivals of one XCD's workgroups, [.. + 1] the
+                              generation its leader passed on, [.. + 2] its workgroups that have finished, [512 + b]
+                              0x100 | the XCC workgroup b ran on (written by the first launch).  A launch leaves
+                              every word but [1], [3] and [512 ..] at zero. */
   int32_t num_instr, layers, d, hq, hkv, dff, vocab, pos, smax, chunks;
   float eps, attn_scale_log2e;
 } MkModel;

@@ -2,15 +2,14 @@
 //
 // One workgroup per CU, all resident at once.  Every workgroup walks the same instruction stream
 // (MkModel.program); an instruction names an op, the op's package does this workgroup's share of it.
-// Where an instruction asks for it, the workgroups meet at a grid barrier: a counter in global memory
-// that only grows, so that what one workgroup wrote (on any XCD) before it is what the others read after it.
+// Where an instruction asks for it, the workgroups meet at a grid barrier: counters in global memory that
+// grow through the launch, so that what one workgroup wrote (on any XCD) before it is what the others read after it.
 // The barrier is in two halves.  A workgroup arrives as soon as its op is done and goes on into the next op, which
 // first asks memory for what no workgroup writes (its first rows of weights, its stretch of the cache) and only
 // then calls back (channel inputs_<op>) to wait for the others: the barrier's 2.5 us and the first loads' latency
 // run side by side.  A normalisation instruction is held back in the same way and runs inside that call.
-// The wait is a bounded poll: a workgroup that gives up raises the status word and goes on without waiting for any
-// further barrier of the launch, and so does every workgroup that sees the word raised: a launch never spins for
-// ever, and one that cannot complete its barriers ends within a few give-up periods.
+// The wait is a bounded poll: a workgroup that gives up raises the status word and goes on; a launch never spins
+// for ever, and one that cannot complete its barriers ends in well under a second.
 #include <pipelink/stage.hpp>
 #ifndef PIPELINK_EMIT
 #include "mk_device.hpp"
@@ -36,10 +35,14 @@ extern "C" __device__ int pipelink_mk_opcode_lmhead();
 
 namespace mk_interp {
 // A wait that is not answered within this many polls is given up.  A barrier takes about 2.5 us, a poll a fraction of a
-// microsecond to a microsecond: 2^16 polls are some tens of milliseconds, thousands of barriers' worth, and short
-// enough that a launch whose workgroups cannot all be resident ends as an error instead of looking like a hang.
-constexpr uint32_t SPIN_LIMIT = 1u << 16;
-constexpr uint32_t STATUS_EVERY = 256;  // a waiting workgroup looks at the status word every so many polls
+// microsecond to a microsecond: 2^13 polls are 5 to 8 ms, two thousand barriers' worth.  A launch whose barriers cannot
+// complete (more workgroups than can be resident, CUs held by another process) gives up each of its 80 waits after
+// that long and ends, with its status word raised, in well under a second.  Making the first give-up final for the
+// workgroup would end it sooner, but every way of remembering it across the ops -- a field of MkPending, a bit of its
+// barrier word, a note in LDS consulted in the poll loop, a look at the status word every 256 polls -- made the step
+// 6 to 25 us slower (the ops have no register to spare, and the poll loop no instruction), so the bound is kept by
+// the limit alone.
+constexpr uint32_t SPIN_LIMIT = 1u << 13;
 constexpr uint32_t STATUS_GAVE_UP = 1u;
 
 // Arrival and release are both in two levels.  An atomic or a load that every XCD must agree on is performed at
@@ -51,19 +54,25 @@ constexpr uint32_t STATUS_GAVE_UP = 1u;
 // workgroups hand each other across a barrier is stored and loaded at device scope (mk::shared_store / shared_load),
 // and every wave has waited for its stores (the __syncthreads) before its workgroup is counted.
 //
-// Every counter only grows, from launch to launch: barrier number g of a launch is generation base + g, where base
-// (sync[3]) is the number of barriers all earlier launches passed.  So no word is ever put back to zero, and each
-// word is only ever touched at one scope: the per-XCD words at workgroup scope by that XCD's workgroups, the grid's
-// words at device scope.  (Unsigned wrap-around is harmless: targets are compared by difference or for equality.)
+// Counters grow through a launch (barrier g of the launch is generation g) and are put back to zero at its end by
+// whoever may touch them: every word is only ever accessed at one scope.  An XCD's words (arrivals, generation,
+// finished) are accessed at workgroup scope by that XCD's workgroups, and the last of them to finish zeroes them;
+// the grid's words at device scope, and the last workgroup of the grid zeroes those.  So a launch needs no memset
+// and no word is ever written from two scopes (a device-scope store to a word that another XCD's L2 holds modified
+// could be undone by that line's write-back).
 //
-// The round-robin assumption is recorded, not trusted blindly: every workgroup ORs the bit of the XCC it really runs
-// on (hardware register XCC_ID) into sync[288 + blockIdx % 8]; the host checks after a launch that each of these
-// words names one XCC and no two name the same (host/megakernel.py raise_on_status).
+// The round-robin assumption is recorded, not trusted blindly: in a session's first launch (sync[3] still zero) every
+// workgroup stores the XCC it really runs on (hardware register XCC_ID) into a word of its own, sync[512 + blockIdx];
+// the host checks that the workgroups with one blockIdx % 8 all ran on one XCC and no two such groups on the same
+// (host/megakernel.py raise_on_status).  (One word per workgroup, a plain store, one launch: 256 device-scope atomics
+// on one line in every launch cost 8 us per token.)
 constexpr int NUM_XCD = 8;
-constexpr int XCD_COUNTER = 32;      // sync[32 * (1 + xcd)]: arrivals; [32 * (1 + xcd) + 1]: generation; one 128-byte line per XCD
-constexpr int XCC_SEEN = 32 * 9;     // sync[288 + xcd]: bits of the XCCs its workgroups ran on (device scope, a line of its own)
-// false: the wait was given up -- by this workgroup now (it then raises the status word), or by any workgroup before
-// (the status word is sticky; the host clears it)
+constexpr int XCD_COUNTER = 32;      // sync[32 * (1 + xcd)]: arrivals; [.. + 1]: generation; [.. + 2]: finished; one 128-byte line per XCD
+constexpr int XCC_SEEN = 512;        // sync[512 + blockIdx]: XCC_RECORDED | the XCC that workgroup ran on
+constexpr int XCC_WORDS = 512;
+constexpr uint32_t XCC_RECORDED = 0x100u;
+// false: the wait was given up (the status word is raised then; it is sticky, the host clears it).  The loop looks at
+// nothing but the word it waits for: a look at the status word as well, even one in 256 polls, cost 6-11 us per token.
 __device__ __forceinline__ bool poll(uint32_t* word, uint32_t target, bool local, const MkModel& m) {
   for (uint32_t spin = 0; spin < SPIN_LIMIT; ++spin) {
     // local: an atomic add of 0 written out as such -- atomics are performed in the L2, whereas a plain
@@ -82,15 +91,12 @@ __device__ __forceinline__ bool poll(uint32_t* word, uint32_t target, bool local
       seen = later;
     }
     if ((int32_t)(seen - target) >= 0) return true;
-    if ((spin & (STATUS_EVERY - 1)) == STATUS_EVERY - 1 &&
-        __hip_atomic_load(m.sync + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
-      return false;  // somebody gave up: this barrier will not complete either
     __builtin_amdgcn_s_sleep(1);
   }
   __hip_atomic_fetch_or(m.sync + 1, STATUS_GAVE_UP, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return false;
 }
-// first half of the barrier of generation `generation` (base + 1, base + 2, ...): this workgroup has finished what comes before it
+// first half of barrier number `generation` (1, 2, ...) of the launch: this workgroup has finished what comes before it
 __device__ __forceinline__ void grid_arrive(const MkModel& m, uint32_t generation) {
   __syncthreads();  // every wave's stores have been issued and acknowledged by the L2
   if (threadIdx.x == 0) {
@@ -101,23 +107,22 @@ __device__ __forceinline__ void grid_arrive(const MkModel& m, uint32_t generatio
       __hip_atomic_fetch_add(m.sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
-// second half: every workgroup has arrived at the barrier of generation pending->barrier.  After a give-up (its own or
-// one it noticed) a workgroup waits for no barrier of the launch any more: the step's results are void by then, and
-// the launch should end quickly.
+// second half: every workgroup has arrived at barrier number pending->barrier.  After a give-up a workgroup waits for
+// no barrier of the launch any more: the step's results are void by then, and the launch should end quickly.  (The others waiting at that barrier give up within the same
+// period; a workgroup that was not running finds every barrier complete when it gets there, because arrivals go on.)
 __device__ __forceinline__ void grid_wait(const MkModel& m, MkPending* pending) {
-  if (threadIdx.x == 0 && !pending->gave_up) {
-    const uint32_t generation = pending->barrier;
+  const uint32_t generation = pending->barrier;
+  if (threadIdx.x == 0) {
     const uint32_t xcd = blockIdx.x % NUM_XCD, groups = min((uint32_t)NUM_XCD, gridDim.x);
     uint32_t* mine = m.sync + XCD_COUNTER * (1 + xcd);
-    bool ok;
     if (blockIdx.x < NUM_XCD) {  // this XCD's first workgroup listens for the grid
-      ok = poll(m.sync, generation * groups, false, m);
+      poll(m.sync, generation * groups, false, m);
       __hip_atomic_exchange(mine + 1, generation, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     } else {
-      ok = poll(mine + 1, generation, true, m);
+      poll(mine + 1, generation, true, m);
     }
-    if (!ok) pending->gave_up = 1;
   }
+  pending->barrier = 0;
   __syncthreads();
 }
 }  // namespace mk_interp
@@ -125,10 +130,7 @@ __device__ __forceinline__ void grid_wait(const MkModel& m, MkPending* pending) 
 // The ops' way to their inputs: the open barrier, then the normalisation that is due.
 __device__ __forceinline__ void mk_interp_inputs(const void* view, MkPending* pending) {
   const MkModel& m = *static_cast<const MkModel*>(static_cast<const pipelink_host_view*>(view)->residue);
-  if (pending->waiting) {
-    mk_interp::grid_wait(m, pending);
-    pending->waiting = 0;
-  }
+  if (pending->barrier != 0) mk_interp::grid_wait(m, pending);
   if (pending->norm != nullptr) {
     pipelink_call_op_rmsnorm(view, pending->norm);
     pending->norm = nullptr;
@@ -151,15 +153,14 @@ extern "C" __device__ void mk_interp_role_worker(const void* params, unsigned va
   (void)variant;
   const MkModel& m = *static_cast<const MkModel*>(params);
   const pipelink_host_view view{params, nullptr};
-  // generations go on from where the launch before stopped
-  const uint32_t base = __hip_atomic_load(m.sync + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  uint32_t passed = base;
-  MkPending pending{nullptr, 0, 0, 0};
-  if (threadIdx.x == 0) {
-    // XCC_ID is bits 3:0 of hardware register 20: s_getreg_b32 with size 4, offset 0
+  uint32_t passed = 0;
+  MkPending pending{nullptr, 0};
+  if (threadIdx.x == 0 && blockIdx.x < mk_interp::XCC_WORDS &&
+      __hip_atomic_load(m.sync + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) {
+    // the session's first launch records where its workgroups run (the dispatch pattern does not change from launch
+    // to launch).  XCC_ID is bits 3:0 of hardware register 20: s_getreg_b32 with size 4, offset 0
     const uint32_t xcc = (uint32_t)__builtin_amdgcn_s_getreg((3 << 11) | 20) & 0xFu;
-    __hip_atomic_fetch_or(m.sync + mk_interp::XCC_SEEN + blockIdx.x % mk_interp::NUM_XCD, 1u << xcc, __ATOMIC_RELAXED,
-                          __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(m.sync + mk_interp::XCC_SEEN + blockIdx.x, mk_interp::XCC_RECORDED | xcc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   for (int i = 0; i < m.num_instr; ++i) {
     const MkInstr* instr = m.program + i;
@@ -182,19 +183,27 @@ extern "C" __device__ void mk_interp_role_worker(const void* params, unsigned va
     if (instr->barrier_after) {
       mk_interp::grid_arrive(m, ++passed);
       pending.barrier = passed;
-      pending.waiting = 1;
     } else {
       __syncthreads();  // the next op of this workgroup reads what this one left in LDS
     }
   }
   mk_interp_inputs(&view, &pending);
-  // The last workgroup to get here records where the next launch's generations start: by then every workgroup has
-  // read this launch's base and left its last barrier.  (Every workgroup arrives at every barrier, waited for or
-  // not, so the counters stay in step with the generation even after a give-up.)
+  // Every workgroup has left its last barrier of the launch when it gets here (it arrives at every barrier, waited for
+  // or not, so the counts are whole even after a give-up).  The last of an XCD's workgroups puts that XCD's words back
+  // to zero, the last of the grid the grid's words: each at the scope the words are used at.
   if (threadIdx.x == 0) {
+    const uint32_t xcd = blockIdx.x % mk_interp::NUM_XCD;
+    const uint32_t members = (gridDim.x - xcd + mk_interp::NUM_XCD - 1) / mk_interp::NUM_XCD;
+    uint32_t* mine = m.sync + mk_interp::XCD_COUNTER * (1 + xcd);
+    if (__hip_atomic_fetch_add(mine + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == members - 1) {
+      __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_store(mine + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_store(mine + 2, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
     const uint32_t before = __hip_atomic_fetch_add(m.sync + 2, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
     if (before == gridDim.x - 1) {
-      __hip_atomic_store(m.sync + 3, passed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(m.sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_fetch_add(m.sync + 3, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // launches closed
       __hip_atomic_store(m.sync + 2, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     }
   }

@@ -157,8 +157,9 @@ def test_host_refuses_grids_that_cannot_be_resident_and_reads_the_status_words(e
     be = _HostMemory(32)
     sess = open_session(*args, workgroups=32, **cfg, backend=be, image=image)
     try:
-        good = np.zeros(512, dtype=np.uint32)
-        good[288:296] = [1 << ((3 * i) % 8) for i in range(8)]      # any permutation of the XCCs will do
+        good = np.zeros(1024, dtype=np.uint32)
+        good[3] = 1                                                 # one launch has closed
+        good[512:512 + 32] = [0x100 | ((3 * (b % 8)) % 8) for b in range(32)]   # any permutation of the XCCs will do
         sess.write("sync", good)
         assert np.array_equal(raise_on_status(sess), good)
         gave_up = good.copy()
@@ -172,7 +173,7 @@ def test_host_refuses_grids_that_cannot_be_resident_and_reads_the_status_words(e
         sess.write("sync", open_launch)
         with pytest.raises(RuntimeError, match="finished"):
             raise_on_status(sess)
-        for bad in ((288, 0b11), (289, 1), (290, 0)):               # two XCCs in one group, one XCC in two groups, none recorded
+        for bad in ((512 + 8, 0x101), (512 + 1, 0x100), (512 + 2, 0)):   # two XCCs in one group, one XCC in two groups, none recorded
             words = good.copy()
             words[bad[0]] = bad[1]
             sess.write("sync", words)
@@ -214,24 +215,16 @@ def _run(paths_key, cfg, weights, cache, x, workgroups, image_key=None, time_lau
 
 
 def _check_sync(sync, workgroups, barriers, launches):
-    """Every word of the barrier's state after `launches` launches: the counters only
-    grow, so a lost arrival, a generation that was not passed on or a launch that did not close shows as a wrong number."""
-    assert sync[1] == 0 and sync[2] == 0
-    assert sync[3] % barriers == 0
-    n = int(sync[3]) // barriers
-    assert n == launches
-    groups = min(8, workgroups)
-    assert sync[0] == n * barriers * groups
-    for xcd in range(groups):
-        members = (workgroups - xcd + 7) // 8
-        assert sync[32 * (1 + xcd)] == n * barriers * members and sync[32 * (1 + xcd) + 1] == n * barriers, xcd
-    seen = [int(w) for w in sync[288:288 + groups]]
-    assert all(w and not w & (w - 1) for w in seen) and len(set(seen)) == groups, seen   # one XCC each, all different
-    rest = np.ones(512, dtype=bool)
-    rest[[0, 1, 2, 3]] = False
-    for xcd in range(8):
-        rest[[32 * (1 + xcd), 32 * (1 + xcd) + 1, 288 + xcd]] = False
-    assert not sync[rest].any()
+    """Every word of the barrier's state after `launches` launches: a launch leaves its counters at zero (each put back
+    at the scope it is used at), counts itself in word 3, and the first one recorded where the workgroups ran."""
+    assert barriers > 0
+    assert sync[0] == 0 and sync[1] == 0 and sync[2] == 0 and sync[3] == launches
+    assert not sync[4:512].any()                                  # the per-XCD arrivals, generations and finished counts
+    ran_on = [int(w) for w in sync[512:512 + workgroups]]
+    assert all(w & 0x100 for w in ran_on)
+    groups = [set(ran_on[x::8]) for x in range(min(8, workgroups))]
+    assert all(len(g) == 1 for g in groups) and len(set.union(*groups)) == len(groups), groups   # one XCC each, all different
+    assert not sync[512 + workgroups:].any()
 
 
 def _rel(a, b):
