@@ -74,7 +74,11 @@ int plk_mok_session_destroy(plk_mok_session* s);
  * the device: a call with the same problem only launches (and can be captured into a graph); a call with another
  * problem first uploads its image, which synchronises the stream -- on a stream that is being captured that call
  * returns PLK_E_CONTRACT.  A problem with more routed-row tiles than any before also makes the session replace its
- * launch workspace (device synchronisation, same rule under capture). */
+ * launch workspace (device synchronisation, same rule under capture).
+ * The one-launch forward counts on its workgroups (one per CU) all running at once, and its counters belong to the
+ * session: forwards of one session must not overlap (one stream, or streams ordered by events), and a forward launched
+ * while another kernel holds CUs may see a down tile give up its bounded wait -- plk_mok_status tells; plk_mok_forward_pass
+ * 1 then 2 has no such dependency inside a launch. */
 int plk_mok_forward(plk_mok_session* s, const plk_mok_problem* p, void* stream);
 int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass, void* stream);
 
