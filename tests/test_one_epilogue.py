@@ -126,24 +126,27 @@ def _bits(t: torch.Tensor) -> np.ndarray:
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("size", [512, 8192])
+@pytest.mark.parametrize("size", [512, (768, 384, 1088), 8192], ids=str)
 def test_three_homes_one_epilogue_bit_exact_and_within_the_bf16_bar(size):
+    """Square sizes, and one where m, n and k all differ (three row tiles of the wide trio, three column tiles, an odd
+    number of ring stages)."""
     from pipelink_amd.host.one_epilogue import open_session
 
-    a, b, scale, bias = gg.scale_bias_inputs(size, size, size, seed=0)
+    m, n, k = size if isinstance(size, tuple) else (size, size, size)
+    a, b, scale, bias = gg.scale_bias_inputs(m, n, k, seed=0)
     a_bits, bt_bits = _bits(a), _bits(b.t())
     results = {}
     for home in oe_build.HOMES + (oe_build.WIDE,):
         paths = oe_build.images(home)
         sess = open_session(paths["link_json"], home, a_bits, bt_bits, bias.numpy(), scale.numpy())
         try:
-            print(f"home {home} size {size}", flush=True)
+            print(f"home {home} m {m} n {n} k {k}", flush=True)
             sess.launch()
             sess.synchronize()
             assert sess.read("status")[0] == 0, "a ring wait gave up"
             results[home] = sess.read("c")
             control = sess.with_image(paths["one_unit"])
-            sess.write("c", np.full((size, size), 0x7FC0, dtype=np.uint16))    # bf16 NaN
+            sess.write("c", np.full((m, n), 0x7FC0, dtype=np.uint16))    # bf16 NaN
             control.launch()
             control.synchronize()
             assert sess.read("status")[0] == 0
@@ -153,7 +156,7 @@ def test_three_homes_one_epilogue_bit_exact_and_within_the_bf16_bar(size):
     assert np.array_equal(results["agpr"], results["vgpr"]) and np.array_equal(results["agpr"], results["lds"])
     # the wide tile multiplies the same 16-element steps in the same order: the same bits
     assert np.array_equal(results["agpr"], results["wide"])
-    rows = torch.arange(size) if size <= 512 else torch.from_numpy(np.random.default_rng(0).choice(size, 48, replace=False))
+    rows = torch.arange(m) if m <= 768 else torch.from_numpy(np.random.default_rng(0).choice(m, 48, replace=False))
     want = gg.gemm_scale_bias_torch(a, b, scale, bias, rows).float().numpy()
     got = torch.from_numpy(results["agpr"].view(np.int16)).view(torch.bfloat16).float().numpy()[rows.numpy()]
     assert np.isfinite(got).all()
