@@ -244,6 +244,45 @@ def cpu_baseline(inp, row_major, slice_tokens=1024):
                       "ms_per_forward": round(sec_slice * 1e3), "runs": "median of 3 after 1 warm-up"}}
 
 
+def vendor_dense_fp8(inp, row_major, torch, ramp_seconds):
+    """What the vendor library's dense FP8 GEMM (`torch._scaled_mm`, one scale per tensor, bf16 out) reaches on this
+    board at the two GEMM shapes of the forward, on the forward's own e4m3 codes: the 32768 routed rows against
+    ONE expert's weights (gate and up stacked; down), so no grouping, no block scales, no activation between the two,
+    and 17 MB + 8 MB of weights instead of 531 MB + 265 MB.  Sustained the same way as the forward, with the board's
+    power and clock beside each.  Best effort: null where the library has no such kernel."""
+    fp8 = torch.float8_e4m3fn
+    x = inp["x_q"][inp["row_token"].long()][:, :H].contiguous().view(fp8)
+    one = torch.ones((), device=x.device)
+    out = {"definition": "torch._scaled_mm(x8, w8.t(), scale_a=1, scale_b=1, out_dtype=bf16), dense, one expert's weights",
+           "operands": "the forward's own e4m3 codes (gathered routed rows; expert 0)"}
+    shapes = (("gate_up", torch.cat([row_major["w_gate_q"][0], row_major["w_up_q"][0]]).contiguous().view(fp8), FLOPS_GATE_UP),
+              ("down", row_major["w_down_q"][0].contiguous().view(fp8), FLOPS_DOWN))
+    try:
+        for name, w, flop in shapes:
+            def run(n):
+                for _ in range(n):
+                    torch._scaled_mm(x, w.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+            end = time.perf_counter() + ramp_seconds
+            while time.perf_counter() < end:
+                run(20)
+                torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            n = 200
+            with PowerSampler() as power:
+                e0.record()
+                run(n)
+                e1.record()
+                torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / n
+            rep = power.report()
+            out[name] = {"m": int(x.shape[0]), "n": int(w.shape[0]), "k": int(w.shape[1]), "ms": round(ms, 4),
+                         "tflops": round(flop / (ms * 1e-3) / 1e12, 1), "draw_w": rep["draw_w"], "sclk_mhz": rep["sclk_mhz"]}
+        out["ms_both"] = round(out["gate_up"]["ms"] + out["down"]["ms"], 4)
+    except Exception as ex:  # noqa: BLE001 -- a library without the kernel, not a failure of this bench
+        out["error"] = repr(ex)[:200]
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -255,6 +294,8 @@ def main() -> int:
     ap.add_argument("--no-pair", action="store_true", help="skip the linked vs one-unit paired timing")
     ap.add_argument("--no-mfma-ceiling", action="store_true",
                     help="skip the pure-MFMA run that measures what the matrix pipe sustains at the board's power limit")
+    ap.add_argument("--vendor-gemm", action="store_true",
+                    help="also time the vendor library's dense FP8 GEMM at the forward's two GEMM shapes (vendor_dense_fp8)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 1 GiB device copy, 10 times: the known-size kernel the FETCH_SIZE / "
                          "WRITE_SIZE counters are scaled by")
@@ -407,6 +448,8 @@ def main() -> int:
         out["mfma_ceiling"] = ceiling
         rnd = ceiling["random_operands"]["tflops"]
         out["roofline"]["frac_of_measured_mfma_ceiling"] = round(FLOPS_TOTAL / (ms_launch * 1e-3) / 1e12 / rnd, 4)
+    if args.vendor_gemm:
+        out["vendor_dense_fp8"] = vendor_dense_fp8(inp, row_major, torch, args.ramp_seconds)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(inp, row_major)
     print(json.dumps(out))
