@@ -22,7 +22,9 @@ def open_session(link_json: str | Path, home: str, a_bits: np.ndarray, bt_bits: 
     n, k2 = bt_bits.shape
     if k != k2 or bias.shape != (n,) or scale.shape != (n,):
         raise ValueError("operand shapes do not agree")
-    tile_m, tile_n = (256, 128) if home == "wide" else (TILE, TILE)
+    tile_m, tile_n = {"wide": (256, 128), "full": (256, 256)}.get(home, (TILE, TILE))
+    if home == "full" and (k < 256 or m * k >= 2 ** 31 or n * k >= 2 ** 31):
+        raise ValueError("the 256 x 256 tile needs k >= 256 and operands below 2^31 elements")
     if m % tile_m or n % tile_n or k % TILE_K or a_bits.dtype != np.uint16 or bt_bits.dtype != np.uint16:
         raise ValueError(f"m must be a multiple of {tile_m}, n of {tile_n}, k of 64, operands uint16 bf16 bit patterns")
     buffers = {"a": a_bits, "bt": bt_bits, "bias": bias.astype(np.float32), "scale": scale.astype(np.float32),

@@ -3,7 +3,9 @@ three-package GEMM example, unchanged), three matrix packages that keep their ac
 VGPRs and in an LDS tile, and ONE epilogue package; links the epilogue against each producer in turn
 (the linker generates the accumulator import for each home) and builds each pipeline's one-unit control.
 A fourth pipeline, ``wide``, is the same composition at the tile size the accumulation registers allow
-(256 x 128 per workgroup, 128 x 64 per wave): its own loader, matrix and epilogue packages.
+(256 x 128 per workgroup, 128 x 64 per wave) that loader waves leave room for: its own loader, matrix and epilogue
+packages.  A fifth, ``full``, is the 256 x 256 tile that takes all of a SIMD's registers: a matrix package whose waves
+load their own operands, and its epilogue.
 
 Counterpart of examples/one-epilogue-many-producers/build.py in the reference.  Output under
 ``build/``: the ``.plink`` packages and, per home (and ``wide``), ``<home>/{pipeline.json, link/..., one_unit.hsaco}``."""
@@ -18,14 +20,21 @@ HERE = Path(__file__).resolve().parent
 BUILD = HERE / "build"
 HOMES = ("agpr", "vgpr", "lds")
 WIDE = "wide"   # the 256 x 128 tile: its own loader, matrix and epilogue packages (accumulator in 128 AGPRs)
+FULL = "full"   # the 256 x 256 tile: a matrix package that loads its own operands, and its epilogue (256 AGPRs)
+CELLS = HOMES + (WIDE, FULL)
 PACKAGES = [("gs.loader", HERE.parent / "gemm_split" / "loader.hip"), ("oe.mma.agpr", HERE / "mma_agpr.hip"),
             ("oe.mma.vgpr", HERE / "mma_vgpr.hip"), ("oe.mma.lds", HERE / "mma_lds.hip"), ("oe.epilogue", HERE / "epilogue.hip"),
             ("oe.loader.wide", HERE / "loader_wide.hip"), ("oe.mma.wide", HERE / "mma_wide.hip"),
-            ("oe.epilogue.wide", HERE / "epilogue_wide.hip")]
+            ("oe.epilogue.wide", HERE / "epilogue_wide.hip"),
+            ("oe.mma.full", HERE / "mma_full.hip"), ("oe.epilogue.full", HERE / "epilogue_full.hip")]
 
 
 def _stages_of(cell_name: str) -> tuple[str, ...]:
-    return ("oe.loader.wide", "oe.mma.wide", "oe.epilogue.wide") if cell_name == WIDE else ("gs.loader", f"oe.mma.{cell_name}", "oe.epilogue")
+    if cell_name == WIDE:
+        return ("oe.loader.wide", "oe.mma.wide", "oe.epilogue.wide")
+    if cell_name == FULL:
+        return ("oe.mma.full", "oe.epilogue.full")
+    return ("gs.loader", f"oe.mma.{cell_name}", "oe.epilogue")
 
 
 def build(out: Path = BUILD, one_unit: bool = True) -> dict:
@@ -34,7 +43,7 @@ def build(out: Path = BUILD, one_unit: bool = True) -> dict:
     out.mkdir(parents=True, exist_ok=True)
     reports = {sid: pack.pack_stage(src, out / f"{sid}.plink") for sid, src in PACKAGES}
     links, controls = {}, {}
-    for home in HOMES + (WIDE,):
+    for home in CELLS:
         cell = out / home
         cell.mkdir(exist_ok=True)
         for sid in _stages_of(home):
@@ -63,5 +72,5 @@ if __name__ == "__main__":
     from pipelink_amd.stages.one_epilogue.build import build as _build
 
     res = _build()
-    print(json.dumps({h: {"depth": l["bindings"]["pipelink_gs_depth"], "dyn_smem_bytes": l["dyn_smem_bytes"],
+    print(json.dumps({h: {"depth": l["bindings"].get("pipelink_gs_depth"), "dyn_smem_bytes": l["dyn_smem_bytes"],
                           "tensor_plans": l["tensor_plans"], "observed": l["observed"]} for h, l in res["links"].items()}, indent=1))

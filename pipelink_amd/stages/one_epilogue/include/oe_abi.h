@@ -24,6 +24,10 @@
 #define OE_WIDE_STAGE_BYTES ((256 + 128) * 128) /* 64 contraction elements of 256 A rows, then of 128 B^T rows */
 #define OE_WIDE_LOAD_WAVES 3                    /* 128 rows each: upper A, lower A, B^T */
 
+/* the 256 x 256 pair (oe.mma.full, which brings its own operands, and oe.epilogue.full): a wave's share 128 x 128 */
+#define OE_FULL_TILE 256
+#define OE_FULL_BUFFERS 5 /* 16 KB buffers (32 contraction elements of 256 rows) per operand ring */
+
 typedef struct OeMmaParams {
   uint32_t* status;
   int32_t n, k;
@@ -48,5 +52,14 @@ typedef struct OeLoaderParams {
   int32_t m, n, k;    /* multiples of 256, 128, 64 */
   int32_t reserved;
 } OeLoaderParams;
+
+/* params of oe.mma.full: operands and extents */
+typedef struct OeFullParams {
+  const uint16_t* a;  /* [M, K] bf16 */
+  const uint16_t* bt; /* [N, K] bf16 */
+  uint32_t* status;   /* [1]; this package has no wait that can give up and leaves it alone */
+  int32_t m, n, k;    /* m, n multiples of 256; k a multiple of 64, at least 256; m * k and n * k below 2^31 elements */
+  int32_t reserved;
+} OeFullParams;
 
 #endif

@@ -12,6 +12,11 @@ def params_blobs(addr: dict[str, int], m: int, n: int, k: int, home: str) -> dic
             "oe.mma.wide": struct.pack("<Qii", addr["status"], n, k),
             "oe.epilogue.wide": struct.pack("<QQQii", addr["bias"], addr["scale"], addr["c"], m, n),
         }
+    if home == "full":
+        return {
+            "oe.mma.full": struct.pack("<QQQiiii", addr["a"], addr["bt"], addr["status"], m, n, k, 0),
+            "oe.epilogue.full": struct.pack("<QQQii", addr["bias"], addr["scale"], addr["c"], m, n),
+        }
     return {
         "gs.loader": struct.pack("<QQQiiii", addr["a"], addr["bt"], addr["status"], m, n, k, 0),
         f"oe.mma.{home}": struct.pack("<Qii", addr["status"], n, k),

@@ -97,6 +97,24 @@ def test_wide_tile_links_its_own_trio(example):
 
 
 @needs_rocm
+def test_full_tile_links_a_matrix_package_that_loads_its_own_operands(example):
+    """256 x 256 workgroup tiles: four waves with 128 x 128 each in all 256 AGPRs and no loader waves beside them, two
+    rings of five 16 KB buffers (all of the LDS), the accumulator handed over transposed, block by block."""
+    out, res = example
+    full = res["links"]["full"]
+    assert [e["stage_id"] for e in full["params"]["entries"]] == ["oe.mma.full", "oe.epilogue.full"]
+    assert full["threads"] == 4 * 64 and full["dyn_smem_bytes"] == 2 * 5 * 256 * 64 == 160 * 1024
+    plan = full["tensor_plans"][0]
+    assert plan["route"] == "accvgpr_receipt" and plan["function"] == "oe_epilogue_full_import_acc"
+    obs = full["observed"]
+    # one wave per SIMD: the whole register file of a lane, nothing spilled; six steps of 32 MFMAs are written out
+    assert obs["calls"] == 0 and obs["private_segment_fixed_size"] == 0 and obs["agpr_count"] == 256 and obs["vgpr_spill_count"] == 0
+    assert obs["mfma"] == 6 * 32
+    stub = (out / "full" / "link" / "stub.hip").read_text()
+    assert "oe_epilogue_full_import_acc_block(const void* source, int block, float* dest)" in stub
+
+
+@needs_rocm
 def test_rejected_tensor_connections_are_named(example, tmp_path):
     cases = [
         ("vgpr", "oe.mma.vgpr", lambda m: m["tensor"]["exports"][0].update(dtype="f16"), None, "T-CONTRACT",
@@ -126,17 +144,17 @@ def _bits(t: torch.Tensor) -> np.ndarray:
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("size", [512, (768, 384, 1088), 8192], ids=str)
+@pytest.mark.parametrize("size", [512, (768, 512, 1088), 8192], ids=str)
 def test_three_homes_one_epilogue_bit_exact_and_within_the_bf16_bar(size):
-    """Square sizes, and one where m, n and k all differ (three row tiles of the wide trio, three column tiles, an odd
-    number of ring stages)."""
+    """Square sizes, and one where m, n and k all differ (three row tiles of the 256-row tiles, an odd number of
+    ring stages)."""
     from pipelink_amd.host.one_epilogue import open_session
 
     m, n, k = size if isinstance(size, tuple) else (size, size, size)
     a, b, scale, bias = gg.scale_bias_inputs(m, n, k, seed=0)
     a_bits, bt_bits = _bits(a), _bits(b.t())
     results = {}
-    for home in oe_build.HOMES + (oe_build.WIDE,):
+    for home in oe_build.CELLS:
         paths = oe_build.images(home)
         sess = open_session(paths["link_json"], home, a_bits, bt_bits, bias.numpy(), scale.numpy())
         try:
@@ -156,6 +174,8 @@ def test_three_homes_one_epilogue_bit_exact_and_within_the_bf16_bar(size):
     assert np.array_equal(results["agpr"], results["vgpr"]) and np.array_equal(results["agpr"], results["lds"])
     # the wide tile multiplies the same 16-element steps in the same order: the same bits
     assert np.array_equal(results["agpr"], results["wide"])
+    # so does the 256 x 256 tile, with the operands' roles swapped (it accumulates the transpose)
+    assert np.array_equal(results["agpr"], results["full"])
     rows = torch.arange(m) if m <= 768 else torch.from_numpy(np.random.default_rng(0).choice(m, 48, replace=False))
     want = gg.gemm_scale_bias_torch(a, b, scale, bias, rows).float().numpy()
     got = torch.from_numpy(results["agpr"].view(np.int16)).view(torch.bfloat16).float().numpy()[rows.numpy()]
