@@ -241,9 +241,9 @@ def test_stated_case_sampled_heads_one_unit_control_and_output_projection():
     # output projection: y = O . W_o^T, W_o [4096, 4096] from N(0,1) * 0.02, through the linked bf16 GEMM
     g = torch.Generator().manual_seed(1)
     w_o = (torch.randn(HQ * 128, HQ * 128, generator=g) * 0.02).to(torch.bfloat16)     # [out, in]: already "B^T"
-    gemm = oe_build.images("wide")     # the 256 x 128 tile
+    gemm = oe_build.images("full")     # the 256 x 256 tile
     ones, zeros = np.ones(HQ * 128, dtype=np.float32), np.zeros(HQ * 128, dtype=np.float32)
-    proj = open_gemm(gemm["link_json"], "wide", o_bits.reshape(B * S, HQ * 128), _bits(w_o), zeros, ones)
+    proj = open_gemm(gemm["link_json"], "full", o_bits.reshape(B * S, HQ * 128), _bits(w_o), zeros, ones)
     try:
         proj.launch()
         proj.synchronize()

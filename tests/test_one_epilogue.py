@@ -143,6 +143,23 @@ def _bits(t: torch.Tensor) -> np.ndarray:
     return t.contiguous().view(torch.int16).numpy().view(np.uint16)
 
 
+def _print_sustained(sess, home, flop):
+    """Sustained rate of the linked image (printed, not asserted): 100 launches back to back after a 1 s ramp, the
+    median of five such runs, with the board's power and clock sampled meanwhile."""
+    import time
+
+    import bench
+
+    end = time.perf_counter() + 1.0
+    while time.perf_counter() < end:
+        sess.time(50)
+    with bench.PowerSampler() as power:
+        ms = sorted(sess.time(100) for _ in range(5))[2]
+    rep = power.report()
+    print(f"{home}: sustained {ms:.3f} ms = {flop / ms / 1e9:.0f} TFLOP/s at {rep['draw_w']} W of {rep['cap_w']} W, "
+          f"{rep['sclk_mhz']} MHz ({rep['samples']} samples)", flush=True)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("size", [512, (768, 512, 1088), 8192], ids=str)
 def test_three_homes_one_epilogue_bit_exact_and_within_the_bf16_bar(size):
@@ -169,6 +186,8 @@ def test_three_homes_one_epilogue_bit_exact_and_within_the_bf16_bar(size):
             control.synchronize()
             assert sess.read("status")[0] == 0
             assert np.array_equal(sess.read("c"), results[home]), f"{home}: linked and one-unit images differ"
+            if m == 8192 and home in ("agpr", "wide", "full"):
+                _print_sustained(sess, home, 2.0 * m * n * k)
         finally:
             sess.close()
     assert np.array_equal(results["agpr"], results["vgpr"]) and np.array_equal(results["agpr"], results["lds"])
