@@ -180,9 +180,36 @@ def _check_slots(handle: str, depth_ident, pipeline: Pipeline, claims: dict[str,
         _reject(path, "barrier slots extent must equal the ring depth", handle=handle)
 
 
-def expand(channel: Channel, pipeline: Pipeline, stages: list[Stage], seen_inits: dict[tuple, tuple] | None = None
-           ) -> Expansion:
-    """Expand one paired channel or raise ``SolveError`` with ``L-PROTO`` failures."""
+def shared_completion(channels: dict[str, Channel]) -> dict[tuple[str, str], str]:
+    """(channel, side) -> the channel whose barrier side it completes on (``member_of``).
+
+    Several tiles that always arrive together may share one counter: one channel's side is the *root* (it owns the
+    slots and the arrival count, and states the bytes one completion stands for as ``tx_bytes: {"sum": [...]}`` over
+    itself and its members), the others name it with ``member_of`` and state only their own tile.  A member may only
+    name a root: membership does not chain."""
+    member: dict[tuple[str, str], str] = {}
+    for name, ch in channels.items():
+        pp, cp = ch.producer["protocol"], ch.consumer["protocol"]
+        if pp.get("kind") != "mbarrier" or cp.get("kind") != "mbarrier":
+            continue
+        for side in ("full", "empty"):
+            ps, cs = pp.get(side), cp.get(side)
+            if isinstance(ps, dict) and isinstance(cs, dict) and ("member_of" in ps or "member_of" in cs):
+                if ps.get("member_of") != cs.get("member_of") or not isinstance(ps.get("member_of"), str):
+                    _reject(f"channels.{name}.protocol.{side}.member_of", "producer and consumer name different roots")
+                member[(name, side)] = ps["member_of"]
+    for (name, side), root in sorted(member.items()):
+        target = channels.get(root)
+        target_side = target.producer["protocol"].get(side) if target and target.producer["protocol"].get("kind") == "mbarrier" else None
+        if not isinstance(target_side, dict) or (root, side) in member:
+            _reject(f"channels.{root}.protocol.{side}", "member_of may only target a root barrier side", member=name)
+    return member
+
+
+def expand(channel: Channel, pipeline: Pipeline, stages: list[Stage], seen_inits: dict[tuple, tuple] | None = None,
+           channels: dict[str, Channel] | None = None, member: dict[tuple[str, str], str] | None = None) -> Expansion:
+    """Expand one paired channel or raise ``SolveError`` with ``L-PROTO`` failures.  ``channels`` and ``member``
+    (``shared_completion``) are needed by a channel that takes part in a shared completion."""
     name = channel.name
     path = f"channels.{name}"
     pp, cp = channel.producer["protocol"], channel.consumer["protocol"]
@@ -205,8 +232,13 @@ def expand(channel: Channel, pipeline: Pipeline, stages: list[Stage], seen_inits
             spath = f"{path}.protocol.{side}"
             if not isinstance(ps, dict) or not isinstance(cs, dict):
                 _reject(spath, "barrier side is missing")
-            if "member_of" in ps or "member_of" in cs:
-                _reject(spath, "shared-completion barrier sides are not supported on this target")
+            root = (member or {}).get((name, side))
+            if root is None and ("member_of" in ps or "member_of" in cs):
+                _reject(spath, "shared-completion sides need the assembly's other channels to expand")
+            if root is not None:
+                # slots and arrivals are the root's; the member only states its own tile
+                ps = dict(channels[root].producer["protocol"][side], tx_bytes=ps.get("tx_bytes", 0))
+                cs = dict(channels[root].consumer["protocol"][side], tx_bytes=cs.get("tx_bytes", 0))
             if ps.get("slots") != cs.get("slots"):
                 _reject(f"{spath}.slots", "producer and consumer slot handles disagree")
             if ps.get("arrive") != cs.get("arrive"):
@@ -216,9 +248,17 @@ def expand(channel: Channel, pipeline: Pipeline, stages: list[Stage], seen_inits
             if arr.get("by") not in roles:
                 _reject(f"{spath}.arrive.count", "arrive count names a role that is not launched", role=arr.get("by"))
             count = arrive_count(arr.get("count"), roles, wave, f"{spath}.arrive.count")
+            members = sorted(m for (m, sd), r in (member or {}).items() if r == name and sd == side)
             tx = []
             for ep, proto_side in ((channel.producer, ps), (channel.consumer, cs)):
                 t = proto_side.get("tx_bytes", 0)
+                if members or isinstance(t, dict):
+                    # a root: one completion stands for its own tile and every direct member's
+                    if not isinstance(t, dict) or sorted(t.get("sum") or []) != sorted([name] + members):
+                        _reject(f"{spath}.tx_bytes.sum", "root sum must name exactly the root and all direct members",
+                                members=members, actual=t.get("sum") if isinstance(t, dict) else t)
+                    pick = (lambda c: c.producer) if ep is channel.producer else (lambda c: c.consumer)
+                    t = sum(tile_bytes(pick(channels[n] if n != name else channel), f"{spath}.tx_bytes") for n in [name] + members)
                 if t == "tile":
                     t = tile_bytes(ep, f"{spath}.tx_bytes")
                 if type(t) is not int or t < 0:
@@ -247,10 +287,12 @@ def expand(channel: Channel, pipeline: Pipeline, stages: list[Stage], seen_inits
                 _reject(f"channels.{seen_inits[key][0]}.protocol.init",
                         "barrier ring has more than one init owner or materializer", expected=pi, actual=seen_inits[key][1])
             seen_inits.setdefault(key, (name, pi))
+        shared = {sd: r for (m, sd), r in (member or {}).items() if m == name}
         return Expansion(name, kind, tx_full=result["full"][2], tx_empty=result["empty"][2],
                          arrive_full=result["full"][1], arrive_empty=result["empty"][1], init_owner=pi.get("owner"),
                          init_materializer=pi["materializer"], slots=(result["full"][0], result["empty"][0]),
-                         depth=depth_ident if not isinstance(depth_ident, tuple) else depth_ident[1])
+                         depth=depth_ident if not isinstance(depth_ident, tuple) else depth_ident[1],
+                         detail={"member_of": shared} if shared else {})
 
     if kind == "call":
         if pp.get("export") != cp.get("export"):
@@ -296,4 +338,5 @@ def expand(channel: Channel, pipeline: Pipeline, stages: list[Stage], seen_inits
 
 def expand_all(channels: dict[str, Channel], pipeline: Pipeline, stages: list[Stage]) -> list[Expansion]:
     seen: dict[tuple, tuple] = {}
-    return [expand(channels[name], pipeline, stages, seen) for name in sorted(channels)]
+    member = shared_completion(channels)
+    return [expand(channels[name], pipeline, stages, seen, channels, member) for name in sorted(channels)]

@@ -9,7 +9,7 @@ import os
 
 import pytest
 
-from pipelink_amd.pipec import channels, glue, manifest, solver
+from pipelink_amd.pipec import channels, glue, linker, manifest, solver
 from pipelink_amd.pipec.clauses import CLAUSES, ClauseFailure, LinkError, PipeLinkError, SchemaError, SolveError, register_clause
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -75,6 +75,25 @@ def double_barrier_base():
     return root
 
 
+def shared_completion_base():
+    """Three tile channels whose `full` sides complete on one counter: `root` owns it, `member` and `leaf` name it."""
+    names = ("root", "member", "leaf")
+    root_full = {"slots": "pipelink_full", "arrive": {"count": 1, "by": "load"}, "tx_bytes": {"sum": list(names)}}
+    member_full = {"member_of": "root", "tx_bytes": "tile"}
+
+    def eps(direction, role):
+        return [ring_endpoint("root", direction, role, root_full), ring_endpoint("member", direction, role, member_full, shape=(2, 2)),
+                ring_endpoint("leaf", direction, role, member_full, shape=(2, 2))]
+    return {"stages": [stage("alpha.stage", {"load": 4}, endpoints=eps("produce", "load"), claims=copy.deepcopy(RING_CLAIMS)),
+                       stage("beta.stage", {"mma": 4}, endpoints=eps("consume", "mma"))],
+            "pipeline": pipeline(["alpha.stage", "beta.stage"], copy.deepcopy(RING_HANDLES))}
+
+
+def symbols_base():
+    """Two artifacts' tables of strong symbols (what `pipec pack` records from each object file)."""
+    return {"tables": {"alpha.stage": {"strong": ["alpha_stage_entry"]}, "beta.stage": {"strong": ["beta_stage_entry"]}}}
+
+
 def call_base():
     decl = 'extern "C" int beta_stage_compute(int value);'
     caller = 'extern "C" int pipelink_call_invoke(int value);'
@@ -130,7 +149,7 @@ def tensor_base():
 
 
 BASES = {"barrier": barrier_base, "double_barrier": double_barrier_base, "call": call_base, "topology": topology_base,
-         "schema": schema_base, "tensor": tensor_base}
+         "schema": schema_base, "tensor": tensor_base, "shared_completion": shared_completion_base, "symbols": symbols_base}
 
 
 def set_path(root, path, value):
@@ -141,6 +160,13 @@ def set_path(root, path, value):
 
 def run_assembly(raw):
     """Load -> validate -> pair -> expand -> solve, as the linker does before code generation."""
+    if "tables" in raw:  # the link's symbol check alone, on manifests that carry these tables
+        loaded = []
+        for stage_id, table in raw["tables"].items():
+            m = stage(stage_id, {})
+            m["symbols"] = {"defined_strong": list(table["strong"])}
+            loaded.append(manifest.load_stage_manifest(m))
+        return linker.check_symbols(loaded)
     stages = [manifest.load_stage_manifest(s) for s in raw["stages"]]
     if "pipeline" not in raw:
         return
@@ -168,6 +194,16 @@ def test_reference_negative_fixture(path):
     assert any(case["expected_path"] in f.path for f in err.value.failures), [f.path for f in err.value.failures]
     if case.get("expected_message"):
         assert any(case["expected_message"] in f.message for f in err.value.failures)
+
+
+def test_shared_completion_expands_to_one_counter_for_three_tiles():
+    """The root's completion stands for its own tile and both members'; the members ride the root's slots and arrivals."""
+    _, _, _, exps, _ = run_assembly(shared_completion_base())
+    by = {e.channel: e for e in exps}
+    assert by["root"].tx_full == 4 * 4 * 2 + 2 * (2 * 2 * 2) and by["root"].detail == {}
+    for m in ("member", "leaf"):
+        assert by[m].tx_full == 2 * 2 * 2 and by[m].detail == {"member_of": {"full": "root"}}
+        assert by[m].slots == by["root"].slots and by[m].arrive_full == by["root"].arrive_full
 
 
 def gallery():
