@@ -161,10 +161,11 @@ def _print_sustained(sess, home, flop):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("size", [512, (768, 512, 1088), 8192], ids=str)
+@pytest.mark.parametrize("size", [512, (256, 256, 256), (512, 256, 320), (768, 512, 1088), 8192], ids=str)
 def test_three_homes_one_epilogue_bit_exact_and_within_the_bf16_bar(size):
-    """Square sizes, and one where m, n and k all differ (three row tiles of the 256-row tiles, an odd number of
-    ring stages)."""
+    """Square sizes, the shortest contractions the 256 x 256 tile takes (8 and 10 slots of 32 elements: its loop's
+    prologue and tail with one or two steady steps between), and one where m, n and k all differ (three row tiles of
+    the 256-row tiles, an odd number of ring stages)."""
     from pipelink_amd.host.one_epilogue import open_session
 
     m, n, k = size if isinstance(size, tuple) else (size, size, size)
