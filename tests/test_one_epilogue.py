@@ -143,6 +143,22 @@ def _bits(t: torch.Tensor) -> np.ndarray:
     return t.contiguous().view(torch.int16).numpy().view(np.uint16)
 
 
+def test_host_rejects_shapes_a_tile_does_not_handle():
+    """Each cell states its tile: 128 x 128 (the three homes), 256 x 128 (wide), 256 x 256 with a contraction of at
+    least 256 (full); anything else is refused before a buffer is allocated."""
+    from pipelink_amd.host.one_epilogue import open_session
+
+    z = lambda *shape: np.zeros(shape, dtype=np.uint16)
+    f = lambda n: np.zeros(n, dtype=np.float32)
+    bad = [("agpr", 192, 128, 64), ("agpr", 128, 128, 96), ("wide", 128, 128, 64), ("wide", 256, 192, 64),
+           ("full", 256, 384, 256), ("full", 384, 256, 256), ("full", 256, 256, 128), ("full", 256, 256, 288)]
+    for home, m, n, k in bad:
+        with pytest.raises(ValueError):
+            open_session("unused.json", home, z(m, k), z(n, k), f(n), f(n))
+    with pytest.raises(ValueError):
+        open_session("unused.json", "full", z(256, 256), z(256, 512), f(256), f(256))   # contractions differ
+
+
 def _print_sustained(sess, home, flop):
     """Sustained rate of the linked image (printed, not asserted): 100 launches back to back after a 1 s ramp, the
     median of five such runs, with the board's power and clock sampled meanwhile."""
