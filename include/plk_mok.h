@@ -76,15 +76,24 @@ int plk_mok_session_destroy(plk_mok_session* s);
  * returns PLK_E_CONTRACT.  A problem with more routed-row tiles than any before also makes the session replace its
  * launch workspace (device synchronisation, same rule under capture).
  * The one-launch forward counts on its workgroups (one per CU) all running at once, and its counters belong to the
- * session: forwards of one session must not overlap (one stream, or streams ordered by events), and a forward launched
- * while another kernel holds CUs may see a down tile give up its bounded wait -- plk_mok_status tells; plk_mok_forward_pass
- * 1 then 2 has no such dependency inside a launch. */
+ * session: forwards of one session must not overlap (one stream, or streams ordered by events).  A forward launched
+ * while another kernel holds CUs may see a down tile give up its bounded wait: the first wait that gives up takes 2^14
+ * polls (a few tens of milliseconds), every other wait of that launch then ends at once, the launch completes, the call
+ * has long returned PLK_OK, and `y` of that forward is void -- plk_mok_status tells, and from the first give-up it
+ * reports the session runs every later forward as two launches.  A caller that shares the GPU with other work asks for
+ * that from the start: plk_mok_session_launches(s, 2); plk_mok_forward_pass 1 then 2 has no dependency inside a launch
+ * either. */
 int plk_mok_forward(plk_mok_session* s, const plk_mok_problem* p, void* stream);
 int plk_mok_forward_pass(plk_mok_session* s, const plk_mok_problem* p, int pass, void* stream);
+/* How plk_mok_forward and plk_mok_forward_static launch from now on: 1 = one launch whenever hidden_q allows it (the
+ * default), 2 = always pass 1 then pass 2.  No counterpart in the reference, whose cluster launch has no such choice. */
+int plk_mok_session_launches(plk_mok_session* s, int launches);
 
 /* Waits for the stream, then returns and clears the sticky status of the session's launches: 0, or MOK_STATUS_* bits
- * (bit 0: a down tile gave up waiting for its rows of `hidden` after 2^18 polls and multiplied what was there --
- * the outputs of that forward are not to be trusted).  The waits are bounded so that a launch always ends. */
+ * (bit 0: a down tile gave up waiting for its rows of `hidden` after 2^14 polls and multiplied what was there --
+ * the outputs of that forward are not to be trusted; the session switches to two launches per forward).  The waits are
+ * bounded so that a launch always ends.  Forwards through plk_mok_forward_static keep their status in the library's
+ * per-GPU area, which every session on that GPU shares: the session that asks first gets (and clears) the bit. */
 int plk_mok_status(plk_mok_session* s, void* stream, uint32_t* status);
 
 /* plk_mok_forward for callers that cannot allocate or wait: code under HIP graph capture, tight serving loops,

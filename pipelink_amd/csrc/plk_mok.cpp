@@ -31,6 +31,8 @@ struct plk_mok_session {
   int32_t compute_units = 0;
   int device = 0;  // the device that was current when the session was created
   bool used_static = false;  // plk_mok_forward_static has run: the static area's status word counts too
+  uint32_t carried_status = 0;  // status bits of a workspace that has been replaced since: plk_mok_status reports them
+  bool two_launches = false;    // plk_mok_forward runs pass 1 then pass 2 (asked for, or a one-launch forward gave up a wait)
 };
 
 // words the session's first workspace is made for (a problem that needs more gets a larger one)
@@ -75,10 +77,17 @@ static bool stream_is_capturing(void* stream) {
   return stream && hipStreamIsCapturing((hipStream_t)stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusActive;
 }
 
-// (re)places the session's workspace by one of at least `words` zeroed words
+// (re)places the session's workspace by one of at least `words` zeroed words.  Everything the device is doing ends
+// first (launches on any stream may use the old one), and the status bits the old one holds stay with the session.
 static int make_workspace(plk_mok_session* s, int64_t words) {
   if (s->workspace) {
-    int rc = plk_hip_free(s->workspace);
+    if (hipDeviceSynchronize() != hipSuccess) return plk_hip_set_error(PLK_E_RESOURCE, "plk_mok: device synchronisation failed");
+    uint32_t word = 0;
+    int rc = plk_hip_readback(&word, s->workspace + MOK_WS_STATUS * 4, sizeof word, nullptr);
+    if (rc == PLK_OK) {
+      s->carried_status |= word;
+      rc = plk_hip_free(s->workspace);
+    }
     s->workspace = 0;
     s->workspace_words = 0;
     if (rc != PLK_OK) return rc;
@@ -216,8 +225,7 @@ static int forward_launch(plk_mok_session* s, const plk_mok_problem* p, int pass
     if (stream_is_capturing(stream))
       return plk_hip_set_error(PLK_E_CONTRACT, "plk_mok_forward: this problem needs a larger workspace; run the forward once "
                                                "before capturing it into a graph");
-    rc = plk_hip_synchronize(nullptr);
-    if (rc == PLK_OK) rc = make_workspace(s, plk_mok::workspace_words(d));
+    rc = make_workspace(s, plk_mok::workspace_words(d));
     if (rc != PLK_OK) return rc;
   }
   std::vector<unsigned char> image(s->link.params_bytes, 0);
@@ -248,8 +256,8 @@ int plk_mok_forward(plk_mok_session* s, const plk_mok_problem* p, void* stream) 
   int rc = check_problem(p);
   if (rc != PLK_OK) return rc;
   if (p->routed_rows == 0) return PLK_OK;
-  if (plk_mok::one_launch_ok(dims_of(p, 0), p->hidden_q)) return forward_launch(s, p, 0, stream);
-  rc = forward_launch(s, p, 1, stream);  // rows of `hidden` that share cache lines: the launch boundary orders the two GEMMs
+  if (!s->two_launches && plk_mok::one_launch_ok(dims_of(p, 0), p->hidden_q)) return forward_launch(s, p, 0, stream);
+  rc = forward_launch(s, p, 1, stream);  // the launch boundary orders the two GEMMs
   if (rc == PLK_OK) rc = forward_launch(s, p, 2, stream);
   return rc;
 }
@@ -267,8 +275,20 @@ int plk_mok_status(plk_mok_session* s, void* stream, uint32_t* status) {
     if (rc == PLK_OK && other) rc = plk_hip_zero(at, sizeof other, stream);
     word |= other;
   }
+  word |= s->carried_status;
+  s->carried_status = 0;
+  // A wait gave up: the GPU is not this session's alone (or the launch was larger than what can be resident).  From
+  // here on the forward is two launches, which depend on nothing inside a launch.
+  if (word & MOK_STATUS_WAIT_GAVE_UP) s->two_launches = true;
   *status = word;
   return rc;
+}
+
+int plk_mok_session_launches(plk_mok_session* s, int launches) {
+  if (!s) return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok_session_launches: null session");
+  if (launches != 1 && launches != 2) return plk_hip_set_error(PLK_E_ARGUMENT, "plk_mok_session_launches: 1 or 2");
+  s->two_launches = launches == 2;
+  return PLK_OK;
 }
 
 int plk_mok_forward_static(plk_mok_session* s, const plk_mok_problem* p, void* stream) {
@@ -292,7 +312,7 @@ int plk_mok_forward_static(plk_mok_session* s, const plk_mok_problem* p, void* s
 
   // The launches' params images travel as the argument of a small kernel that stores them into the static area and
   // clears the workspace: no copy from host memory, no wait, and stream order puts it in front of the launches.
-  const bool one = plk_mok::one_launch_ok(dims_of(p, 0), p->hidden_q);
+  const bool one = !s->two_launches && plk_mok::one_launch_ok(dims_of(p, 0), p->hidden_q);
   const int passes[2] = {one ? 0 : 1, 2};
   const int launches = one ? 1 : 2;
   StaticImages images;

@@ -78,6 +78,7 @@ SIGNATURES = {
     "plk_mok_forward_pass": (c_int, [c_void_p, POINTER(MokProblem), c_int, c_void_p]),
     "plk_mok_forward_static": (c_int, [c_void_p, POINTER(MokProblem), c_void_p]),
     "plk_mok_status": (c_int, [c_void_p, c_void_p, POINTER(ctypes.c_uint32)]),
+    "plk_mok_session_launches": (c_int, [c_void_p, c_int]),
     "plk_mxfp8_scales_to_slot_major": (c_int, [c_uint64, c_int64, c_int32, c_int32, c_uint64, c_void_p]),
     "plk_mxfp8_codes_to_k64_tiled": (c_int, [c_uint64, c_int64, c_int32, c_int64, c_uint64, c_void_p]),
     "plk_mxfp8_quantize": (c_int, [c_uint64, c_int, c_int64, c_int32, c_uint64, c_int32, c_uint64, c_int32, c_void_p]),

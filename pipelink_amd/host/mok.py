@@ -143,6 +143,11 @@ class MoKSession:
         check(self.lib, self.lib.plk_mok_status(self._handle, s, byref(word)))
         return word.value
 
+    def launches(self, n: int) -> None:
+        """``plk_mok_session_launches``: 1 = one launch per forward whenever ``hidden_q`` allows it (the default), 2 = always
+        gate/up then down as two launches (for a GPU that is shared with other work)."""
+        check(self.lib, self.lib.plk_mok_session_launches(self._handle, n))
+
     def forward_static(self, problem: MokProblem, stream: int | None = None) -> None:
         """Both passes through the entry point that allocates nothing (``plk_mok_forward_static``): the params images
         go into a fixed area of device memory the library owns; calls that overlap on one GPU race on it."""

@@ -68,48 +68,62 @@ __device__ __forceinline__ uint32_t quantise4(float a, float b, float c, float d
   return __builtin_bit_cast(uint32_t, v);
 }
 
-template <bool CLAMPED>
+template <bool CLAMPED, bool SMALL>  // SMALL: a tile of few rows or few columns (mok::tile_placement), else a full tile
 __device__ __forceinline__ void forward(const MokActResidue& p, const MokActTask& t, const AccFrag& acc, const MokCounters& counters) {
   const int tid = fresh_tid();
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int half = lane >> 5;
   unsigned char* stage = pipelink_smem + pipelink_mok_act_arena();
-  // (a wave whose rows or columns all lie past the end computes on an accumulator the GEMM owner
-  // cleared and did not fill; a branch around the arithmetic for it costs every wave spills)
+  // One pair of fragments -- gate values and up values of the same 32 routed rows x 32 columns -> 32 x 32 codes and
+  // 32 scale bytes in the LDS tile; trow = the lane's tile-local routed row, tcol = the block's tile-local first column.
+  auto requantise = [&](const v16f& gate, const v16f& up, int trow, int tcol) {
+    float h[16];
+    float amax = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      h[r] = swiglu<CLAMPED>(gate[r], up[r], p.swiglu_limit);
+      h[r + 1] = swiglu<CLAMPED>(gate[r + 1], up[r + 1], p.swiglu_limit);
+      amax = fmaxf(fmaxf(amax, fabsf(h[r])), fabsf(h[r + 1]));
+    }
+    // the other 16 columns of this row's block live in lane ^ 32
+    amax = fmaxf(amax, __shfl_xor(amax, 32));
+    // The block's scale comes from the largest bf16-rounded magnitude; rounding is monotonic,
+    // so that is the rounded largest magnitude.
+    const f32x2 am = {amax, 0.0f};
+    const uint32_t am_bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(am, bf16x2));
+    int e = (int)((am_bits >> 7) & 0xFFu) - 8;  // floor(log2(amax)) - 8 + 127
+    e = e < 0 ? 0 : e;                          // amax < 2^-118: scale byte 0
+    // 2^(e - 127), a denormal for byte 0; the conversion only looks at the exponent the byte stands for
+    const uint32_t scale_bits = (uint32_t)e << 23;
+    const float scale = __uint_as_float(scale_bits > 0x00400000u ? scale_bits : 0x00400000u);
+    const float limit = __uint_as_float(((uint32_t)(e + 8) << 23) | 0x00600000u);  // 448 * 2^(e - 127), e <= 246
+    unsigned char* dst = stage + trow * STAGE_PITCH + tcol + 4 * half;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      *reinterpret_cast<uint32_t*>(dst + 8 * q) = quantise4(h[4 * q], h[4 * q + 1], h[4 * q + 2], h[4 * q + 3], limit, scale);
+    if (half == 0) stage[STAGE_SCALE_OFF + trow * 4 + (tcol >> 5)] = (uint8_t)e;
+  };
   // ---- activation + requant into an LDS tile [256 rows][128 codes] + [256 rows][4 scales] ----
+  const int placement = tile_placement(t.row_end - t.row_begin, p.cols - t.col_begin);
+  if constexpr (!SMALL) {
+    (void)placement;
+    // (a wave whose rows or columns all lie past the end computes on an accumulator the GEMM owner
+    // cleared and did not fill; a branch around the arithmetic for it costs every wave spills)
 #pragma unroll
-  for (int a = 0; a < 2; ++a) {  // gate fragments a, up fragments a + 2: same rows, same columns
-    const int tcol = wrow0(wave, a);  // tile-local first column of this 32-column block
+    for (int a = 0; a < 2; ++a) {  // gate fragments a, up fragments a + 2: same rows, same columns
 #pragma unroll
-    for (int b = 0; b < XFRAGS; ++b) {
-      const int trow = xrow0(wave, b) + (lane & 31);
-      const v16f gate = from_acc(acc.v[a][b]), up = from_acc(acc.v[a + 2][b]);
-      float h[16];
-      float amax = 0.0f;
+      for (int b = 0; b < XFRAGS; ++b)
+        requantise(from_acc(acc.v[a][b]), from_acc(acc.v[a + 2][b]), xrow0(wave, b) + (lane & 31), wrow0(wave, a));
+    }
+  } else {
+    // a tile of few rows or few columns: 64 routed rows per wave, one or two pairs of fragments (mok::SmallPlacement)
+    const SmallPlacement sp = small_placement(placement, __builtin_amdgcn_readfirstlane(wave));
 #pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        h[r] = swiglu<CLAMPED>(gate[r], up[r], p.swiglu_limit);
-        h[r + 1] = swiglu<CLAMPED>(gate[r + 1], up[r + 1], p.swiglu_limit);
-        amax = fmaxf(fmaxf(amax, fabsf(h[r])), fabsf(h[r + 1]));
-      }
-      // the other 16 columns of this row's block live in lane ^ 32
-      amax = fmaxf(amax, __shfl_xor(amax, 32));
-      // The block's scale comes from the largest bf16-rounded magnitude; rounding is monotonic,
-      // so that is the rounded largest magnitude.
-      const f32x2 am = {amax, 0.0f};
-      const uint32_t am_bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(am, bf16x2));
-      int e = (int)((am_bits >> 7) & 0xFFu) - 8;  // floor(log2(amax)) - 8 + 127
-      e = e < 0 ? 0 : e;                          // amax < 2^-118: scale byte 0
-      // 2^(e - 127), a denormal for byte 0; the conversion only looks at the exponent the byte stands for
-      const uint32_t scale_bits = (uint32_t)e << 23;
-      const float scale = __uint_as_float(scale_bits > 0x00400000u ? scale_bits : 0x00400000u);
-      const float limit = __uint_as_float(((uint32_t)(e + 8) << 23) | 0x00600000u);  // 448 * 2^(e - 127), e <= 246
-      unsigned char* dst = stage + trow * STAGE_PITCH + tcol + 4 * half;
+    for (int b = 0; b < 2; ++b) requantise(from_acc(acc.v[0][b]), from_acc(acc.v[2][b]), sp.xr0 + 32 * b + (lane & 31), sp.wr[0]);
+    if (placement == TILE_SMALL_COLS) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        *reinterpret_cast<uint32_t*>(dst + 8 * q) = quantise4(h[4 * q], h[4 * q + 1], h[4 * q + 2], h[4 * q + 3], limit, scale);
-      if (half == 0) stage[STAGE_SCALE_OFF + trow * 4 + (tcol >> 5)] = (uint8_t)e;
+      for (int b = 0; b < 2; ++b) requantise(from_acc(acc.v[1][b]), from_acc(acc.v[3][b]), sp.xr0 + 32 * b + (lane & 31), sp.wr[1]);
     }
   }
   __syncthreads();
@@ -145,9 +159,12 @@ __device__ __forceinline__ void forward(const MokActResidue& p, const MokActTask
       }
     }
   }
-  // Every wave's stores have completed (the barrier's fence waits for them) before the tile is counted: the row tile's
-  // counter reaches the number of gate/up column tiles when all of its `hidden` is in memory
+  // The tile is counted when all of it is in memory: every wave waits until its own stores above have been written
+  // through (a store leaves the wave's vector-memory count when it is acknowledged; the barrier's workgroup-scope
+  // fence does not wait for that), then the workgroup meets, then one thread counts the tile.  The row tile's counter
+  // reaches the number of gate/up column tiles when all of its `hidden` can be read by any workgroup
   // (campaigns/mok/port/framework/interp_fwd.cu:174-213: the reference's act -> down dependency).
+  if (t.counter_idx >= 0 && counters.base) __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
   __syncthreads();  // also: the staging tile shares LDS with the GEMM ring of the next tile
   if (t.counter_idx >= 0 && counters.base && tid == 0)
     __hip_atomic_fetch_add(counters.base + t.counter_idx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -162,9 +179,21 @@ extern "C" __device__ void mok_act_fwd(const void* view, const MokActTask* task,
   (void)phase;
   const auto& p = *static_cast<const MokActResidue*>(static_cast<const pipelink_host_view*>(view)->residue);
   if (pipelink_mok_clamp())
-    mok_act_owner::forward<true>(p, *task, *acc, *counters);
+    mok_act_owner::forward<true, false>(p, *task, *acc, *counters);
   else
-    mok_act_owner::forward<false>(p, *task, *acc, *counters);
+    mok_act_owner::forward<false, false>(p, *task, *acc, *counters);
+}
+
+// The same for a tile whose accumulator is in the small placement (mok::tile_placement of the task's extent is not
+// TILE_FULL): the caller tells the two apart, as it does for the GEMM owner's exports.
+extern "C" __device__ void mok_act_fwd_small(const void* view, const MokActTask* task, const MokCounters* counters,
+                                             uint32_t* phase, const mok::AccFrag* acc) {
+  (void)phase;
+  const auto& p = *static_cast<const MokActResidue*>(static_cast<const pipelink_host_view*>(view)->residue);
+  if (pipelink_mok_clamp())
+    mok_act_owner::forward<true, true>(p, *task, *acc, *counters);
+  else
+    mok_act_owner::forward<false, true>(p, *task, *acc, *counters);
 }
 #else  // PIPELINK_EMIT: host-evaluated annotations only
 #include "../include/mok_abi.h"
@@ -180,8 +209,12 @@ PL_EXPORT(mok_act_init, mok_act_init, "extern \"C\" __device__ void mok_act_init
 PL_EXPORT(mok_act_fwd, mok_act_fwd,
           "extern \"C\" __device__ void mok_act_fwd(const void* view, const MokActTask* task, "
           "const MokCounters* counters, uint32_t* phase, const mok::AccFrag* acc);");
+PL_EXPORT(mok_act_fwd_small, mok_act_fwd_small,
+          "extern \"C\" __device__ void mok_act_fwd_small(const void* view, const MokActTask* task, "
+          "const MokCounters* counters, uint32_t* phase, const mok::AccFrag* acc);");
 PL_SERVE(act_init, "mok_act_init");
 PL_SERVE(act_fwd, "mok_act_fwd");
+PL_SERVE(act_fwd_small, "mok_act_fwd_small");
 // staging tile for the coalesced write-out; lives while no GEMM ring slot is in use
 PL_CLAIM("pipelink_mok_act_arena", "smem", 256 * 144 + 256 * 4, 1024, "phase:instr_act");
 // host contract (campaigns/mok/port/act/act.cu:280-330 in the reference)

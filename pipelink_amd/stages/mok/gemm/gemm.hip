@@ -329,26 +329,32 @@ __device__ __forceinline__ bool staged_ready(const MokGemmTask& t, const MokCoun
   return *reinterpret_cast<const volatile int32_t*>(r.peek()) >= t.wait_target;
 }
 // Waits until the rows the task reads are complete: one thread polls the counter at device scope, the others wait at
-// the barrier.  A bounded poll: after WAIT_POLLS probes it raises the launch's status word and goes on (the tile then
-// multiplies whatever `hidden` holds), so a launch never spins for ever.
-constexpr uint32_t WAIT_POLLS = 1u << 18;
+// the barrier.  A bounded poll: after WAIT_POLLS probes (a few tens of milliseconds; a wait that can be met takes
+// microseconds) it raises the launch's status word and goes on (the tile then multiplies whatever `hidden` holds), so a
+// launch never spins for ever.  The first wait that gives up also says so in a word of the launch's own, which every
+// waiting thread looks at before it polls and every 256 polls: the launch's results are void by then, and its other
+// waits end at once instead of each running to the limit.
+constexpr uint32_t WAIT_POLLS = 1u << 14;
 __device__ __forceinline__ void wait_rows(const MokGemmTask& t, const MokCounters& counters) {
   if (!waits(t, counters)) return;
   if (threadIdx.x == 0) {
-    bool ok = false;
+    uint32_t* const gave_up = counters.status ? counters.status + (MOK_WS_GAVE_UP - MOK_WS_STATUS) : nullptr;
     uint32_t limit = WAIT_POLLS;
     if (counters.status) {  // the host may shorten the wait (MOK_WS_POLL_LIMIT)
       const uint32_t asked = __hip_atomic_load(counters.status + (MOK_WS_POLL_LIMIT - MOK_WS_STATUS), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (asked != 0) limit = asked;
     }
-    for (uint32_t spin = 0; spin < limit; ++spin) {
-      if (__hip_atomic_load(counters.base + t.counter_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= t.wait_target) {
-        ok = true;
-        break;
-      }
+    bool ok = false;
+    for (uint32_t spin = 0;; ++spin) {
+      ok = __hip_atomic_load(counters.base + t.counter_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= t.wait_target;
+      if (ok || spin >= limit) break;
+      if ((spin & 255u) == 0 && gave_up && __hip_atomic_load(gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
       __builtin_amdgcn_s_sleep(8);
     }
-    if (!ok && counters.status) __hip_atomic_fetch_or(counters.status, (uint32_t)MOK_STATUS_WAIT_GAVE_UP, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!ok && counters.status) {
+      __hip_atomic_fetch_or(counters.status, (uint32_t)MOK_STATUS_WAIT_GAVE_UP, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
   __syncthreads();
 }
@@ -703,6 +709,133 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   wg_barrier();  // every wave holds its last operands in registers: the ring is free
 }
 
+
+// ---- tiles with little to multiply (mok::tile_placement) ----------------------------------------------------------
+// An expert's rows past its last full tile (1 to 64 of them) and the columns past the last full column tile (64 of
+// them when the width is 2880) would keep two of the four waves busy with a 128 x 128 share that is mostly padding,
+// for as long as a full tile takes.  Such a tile is multiplied in the other placement: every wave takes 64 routed
+// rows and one or two pairs of weight fragments, a quarter or half of the full tile's MFMAs spread over all four
+// SIMDs, and the tile takes as long as its loads do.  Rings, loader, waits and barriers are the full tile's (the
+// loader does not know the difference); the loop is the plain two-stage one the full tile ends with.
+struct SmallOperands {
+  v8i x[2], w[4];
+};
+
+template <int DEPTH, int FRAGS>  // FRAGS: the weight fragments that are multiplied, bit a
+__device__ __forceinline__ void mainloop_small(const MokGemmResidue& g, const MokGemmTask& t, int placement, AccFrag& acc,
+                                               const GemmCarry& carry, const MokGemmTask* upcoming, const MokCounters& counters) {
+  const int tid = fresh_tid();  // nothing of this path is to be computed ahead and kept across full tiles
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r32 = lane & 31;
+  const int half = lane >> 5;
+  const Views v = views_of(g, t);
+  const int n = v.act.k / K_SLOT;
+  constexpr int XDEPTH = DEPTH + 1;
+  const Rings<DEPTH> r;
+  const Loader ld = make_loader(v, t, carry);
+  const SmallPlacement sp = small_placement(placement, wave);
+  auto used = [](int a) { return (FRAGS >> a & 1) != 0; };
+
+  int xoff[2], xscoff[2], woff[4], wscoff[4];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const int row = sp.xr0 + 32 * b + r32;
+    xoff[b] = row * K_SLOT + 16 * (half ^ swizzle(row));
+    xscoff[b] = row * 16;
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int wl = sp.wr[a] + r32;
+    woff[a] = wl * K_SLOT + 16 * (half ^ swizzle(wl));
+    wscoff[a] = wl * 4;
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+      if (used(a)) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc.v[a][b][q] = 0.0f;
+      }
+
+  // the prologue of the full tile: steps -DEPTH and 1 - DEPTH were issued by `prefetch`
+#pragma unroll
+  for (int u = 2 - DEPTH; u < 0; ++u) issue_step(ld, r, u, n, (u + DEPTH) & ~1, ((u + DEPTH) & ~1) + 1, u + DEPTH);
+  if (upcoming->op != 0) stage(g, *upcoming, counters);
+  wait_loads_and_reads_dyn(loads_younger_than_slot<DEPTH>(0, -1, n));
+  wg_barrier();
+
+  auto xnext = [](int b, int by) {
+    const int c = b + by;
+    return c >= XDEPTH ? c - XDEPTH : c;
+  };
+  auto read_operands_small = [&](SmallOperands& o, const unsigned char* xbuf, const unsigned char* wbuf) {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) o.x[b] = read_frag(xbuf, xoff[b]);
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+      if (used(a)) o.w[a] = read_frag(wbuf, woff[a]);
+  };
+  // block scales of the pair of slots that starts at slot j (j even), as read_scales does for the full tile
+  auto read_scales_small = [&](int (&sx_)[2], int (&sw_)[4], int j) {
+    const int c = (j & 7) >> 1;
+    const unsigned char* xbuf = r.xscale() + ((j >> 3) & 1) * (TILE_X * 16);
+    const unsigned char* wbuf = r.wscale() + c * (TILE_W * 4);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) sx_[b] = (int)(*reinterpret_cast<const uint32_t*>(xbuf + 4 * c + xscoff[b]) >> (8 * half));
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+      if (used(a)) sw_[a] = (int)(*reinterpret_cast<const uint32_t*>(wbuf + wscoff[a]) >> (8 * half));
+  };
+  SmallOperands even, odd;
+  int sx[2], sw[4], sxn[2], swn[4];
+  auto multiply = [&](auto ODD_, const SmallOperands& o) {
+    constexpr bool ODD = decltype(ODD_)::value;
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+      if (used(a)) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+          acc.v[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.w[a], o.x[b], acc.v[a][b], 0, 0, ODD ? 2 : 0, sw[a],
+                                                                        ODD ? 2 : 0, sx[b]);
+      }
+  };
+  read_operands_small(even, r.x(0), r.w(0));
+  read_scales_small(sx, sw, 0);
+  int xb = 0, wb = 0;
+  auto advance = [&](int t_, SmallOperands& next) {
+    wait_loads_and_reads_dyn(loads_younger_than_slot<DEPTH>(t_ + 1, t_ - 1, n));
+    wg_barrier();
+    const bool odd_step = t_ & 1;
+    issue_step(ld, r, t_, n, odd_step ? xnext(xb, XDEPTH - 2) : xnext(xb, XDEPTH - 1), odd_step ? xnext(xb, XDEPTH - 1) : xb, wb);
+    xb = xnext(xb, 1);
+    wb = wb + 1 == DEPTH ? 0 : wb + 1;
+    read_operands_small(next, r.x(xb), r.w(wb));
+  };
+  int j = 0;
+  for (; j + 1 < n; j += 2) {
+    advance(j, odd);
+    multiply(std::false_type{}, even);
+    advance(j + 1, even);
+    read_scales_small(sxn, swn, j + 2);
+    multiply(std::true_type{}, odd);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) sx[b] = sxn[b];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+      if (used(a)) sw[a] = swn[a];
+  }
+  if (n & 1) multiply(std::false_type{}, even);
+  wg_barrier();  // every wave holds its last operands in registers: the ring is free
+}
+
+// which placement the task's tile has: its routed rows that exist, its output columns that exist
+__device__ __forceinline__ int placement_of(const MokGemmResidue& g, const MokGemmTask& t) {
+  const int cols = (t.op == MOK_GEMM_FWD_ROUTED_GATE_UP ? g.w_gate.rows : g.w_down.rows) - t.col_begin;
+  return tile_placement(t.row_end - t.row_begin, cols);
+}
+
 // bf16 epilogue of the down op.  The accumulator is transposed through the arena buffers (idle
 // by now; the head may already hold the next tile's first slots) so that the global stores
 // are 16 bytes per lane and 512 contiguous bytes per routed row; an arena too small for the
@@ -718,14 +851,38 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // v_cvt_pk_bf16_f32, nearest even
 }
 
-template <int DEPTH>
-__device__ __forceinline__ void store_down(const MokGemmResidue& g, const MokGemmTask& t, const AccFrag& acc) {
+template <int DEPTH, int FRAGS>  // FRAGS: 0 for a full tile, else the fragments a small tile's waves hold
+__device__ __forceinline__ void store_down(const MokGemmResidue& g, const MokGemmTask& t, int placement, const AccFrag& acc) {
   constexpr int ARENA_BYTES = (2 * DEPTH - 3) * BUF_BYTES;
   const int tid = fresh_tid();
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const bool idle = wave_idle(t, g.w_down.rows);  // this wave's accumulator holds nothing
+  constexpr bool small = FRAGS != 0;
+  const SmallPlacement sp = small_placement(placement, __builtin_amdgcn_readfirstlane(wave));
+  const bool idle = !small && wave_idle(t, g.w_down.rows);  // this wave's accumulator holds nothing
   if constexpr (ARENA_BYTES < TILE_X / 2 * Y_PITCH) {
+    if (small) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const int row = t.row_begin + sp.xr0 + 32 * b + (lane & 31);
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          if (!(FRAGS >> a & 1)) continue;
+          const v16f f = from_acc(acc.v[a][b]);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int col = t.col_begin + sp.wr[a] + 8 * q + 4 * (lane >> 5);
+            if (row < t.row_end && col < g.w_down.rows) {
+              uint2 pk;
+              pk.x = pack_bf16x2(f[4 * q + 0], f[4 * q + 1]);
+              pk.y = pack_bf16x2(f[4 * q + 2], f[4 * q + 3]);
+              *reinterpret_cast<uint2*>(g.y + (int64_t)row * g.ld_y + col) = pk;
+            }
+          }
+        }
+      }
+      return;
+    }
     if (idle) return;
 #pragma unroll
     for (int b = 0; b < XFRAGS; ++b) {
@@ -753,7 +910,29 @@ __device__ __forceinline__ void store_down(const MokGemmResidue& g, const MokGem
     const bool col_ok = t.col_begin + chunk * 8 < g.w_down.rows;  // column extents are multiples of 32
 #pragma unroll
     for (int pass = 0; pass < PASSES; ++pass) {
-      if (!idle && (PASSES == 1 || wave_x(wave) == pass)) {
+      if (small) {
+        // every wave's 64 rows lie in one pass; a tile of at most 64 rows has nothing in a second pass
+        if (PASSES == 2 && pass == 1 && placement == TILE_SMALL_ROWS) break;
+        if (PASSES == 1 || (sp.xr0 >= ROWS) == (pass == 1)) {
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            unsigned char* rowp = stage + (sp.xr0 + 32 * b - pass * ROWS + (lane & 31)) * Y_PITCH;
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+              if (!(FRAGS >> a & 1)) continue;
+              const v16f f = from_acc(acc.v[a][b]);
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                const int col = sp.wr[a] + 8 * q + 4 * (lane >> 5);
+                uint2 pk;
+                pk.x = pack_bf16x2(f[4 * q + 0], f[4 * q + 1]);
+                pk.y = pack_bf16x2(f[4 * q + 2], f[4 * q + 3]);
+                *reinterpret_cast<uint2*>(rowp + col * 2) = pk;
+              }
+            }
+          }
+        }
+      } else if (!idle && (PASSES == 1 || wave_x(wave) == pass)) {
 #pragma unroll
         for (int b = 0; b < XFRAGS; ++b) {
           unsigned char* rowp = stage + (xrow0(wave, b) - pass * ROWS + (lane & 31)) * Y_PITCH;
@@ -797,6 +976,11 @@ static __device__ __forceinline__ const MokGemmResidue& mok_gemm_residue(const v
   return *static_cast<const MokGemmResidue*>(static_cast<const pipelink_host_view*>(view)->residue);
 }
 
+// The placement of the task's tile (mok::TILE_FULL, or one of the small ones): which exports the caller uses for it.
+extern "C" __device__ int mok_gemm_placement(const void* view, const MokGemmTask* task) {
+  return mok_gemm_owner::placement_of(mok_gemm_residue(view), *task);
+}
+
 // Looks ahead to a task outside a mainloop (a workgroup's first tile): asks for the task's row tokens and readiness
 // counter.  The caller waits for its loads and passes a workgroup barrier before it calls mok_gemm_ready / _prefetch.
 extern "C" __device__ void mok_gemm_stage(const void* view, const MokGemmTask* task, const MokCounters* counters) {
@@ -810,7 +994,7 @@ extern "C" __device__ bool mok_gemm_ready(const void* view, const MokGemmTask* t
 }
 
 // Waits (bounded) until the rows the task reads are complete; raises MOK_STATUS_WAIT_GAVE_UP in *counters->status
-// if they are not after 2^18 polls.  Must not be called while the workgroup holds a tile whose results others wait for.
+// if they are not after 2^14 polls (or at once, if a wait of the launch has given up before).  Must not be called while the workgroup holds a tile whose results others wait for.
 extern "C" __device__ void mok_gemm_wait(const void* view, const MokGemmTask* task, const MokCounters* counters) {
   (void)view;
   mok_gemm_owner::wait_rows(*task, *counters);
@@ -844,13 +1028,50 @@ extern "C" __device__ void mok_gemm_fwd(const void* view, const MokGemmTask* tas
   ++*phase;
 }
 
+// mok_gemm_fwd for a tile in the small placement (mok::tile_placement of the task's extent is not TILE_FULL): the
+// caller tells the two apart, and hands the accumulator to mok_act_fwd_small / mok_gemm_store_small.
+extern "C" __device__ void mok_gemm_fwd_small(const void* view, const MokGemmTask* task, const MokCounters* counters,
+                                              uint32_t* phase, mok::AccFrag* acc, const mok::GemmCarry* carry,
+                                              const MokGemmTask* upcoming) {
+  const auto& g = mok_gemm_residue(view);
+  const int placement = mok_gemm_owner::placement_of(g, *task);
+  const bool gate_up = task->op == MOK_GEMM_FWD_ROUTED_GATE_UP;
+  const int frags = placement == mok::TILE_SMALL_ROWS ? mok::SMALL_ROWS_FRAGS
+                    : gate_up ? mok::SMALL_COLS_FRAGS_GATE_UP : mok::SMALL_COLS_FRAGS_DOWN;
+#define PL_SMALL(D, F) case F: mok_gemm_owner::mainloop_small<D, F>(g, *task, placement, *acc, *carry, upcoming, *counters); break;
+  switch (pipelink_mok_gemm_depth()) {
+    case 2:
+      switch (frags) { PL_SMALL(2, mok::SMALL_ROWS_FRAGS) PL_SMALL(2, mok::SMALL_COLS_FRAGS_GATE_UP) PL_SMALL(2, mok::SMALL_COLS_FRAGS_DOWN) }
+      break;
+    default:
+      switch (frags) { PL_SMALL(4, mok::SMALL_ROWS_FRAGS) PL_SMALL(4, mok::SMALL_COLS_FRAGS_GATE_UP) PL_SMALL(4, mok::SMALL_COLS_FRAGS_DOWN) }
+      break;
+  }
+#undef PL_SMALL
+  ++*phase;
+}
+
 // Down op only: rounds the accumulator to bf16 and stores the tile of y.
 extern "C" __device__ void mok_gemm_store(const void* view, const MokGemmTask* task, const mok::AccFrag* acc) {
   const auto& g = mok_gemm_residue(view);
   switch (pipelink_mok_gemm_depth()) {
-    case 2: mok_gemm_owner::store_down<2>(g, *task, *acc); break;
-    default: mok_gemm_owner::store_down<4>(g, *task, *acc); break;
+    case 2: mok_gemm_owner::store_down<2, 0>(g, *task, mok::TILE_FULL, *acc); break;
+    default: mok_gemm_owner::store_down<4, 0>(g, *task, mok::TILE_FULL, *acc); break;
   }
+}
+
+// mok_gemm_store for a tile in the small placement.
+extern "C" __device__ void mok_gemm_store_small(const void* view, const MokGemmTask* task, const mok::AccFrag* acc) {
+  const auto& g = mok_gemm_residue(view);
+  const int placement = mok_gemm_owner::placement_of(g, *task);
+#define PL_STORE(D)                                                                                                  \
+  if (placement == mok::TILE_SMALL_ROWS) mok_gemm_owner::store_down<D, mok::SMALL_ROWS_FRAGS>(g, *task, placement, *acc); \
+  else mok_gemm_owner::store_down<D, mok::SMALL_COLS_FRAGS_DOWN>(g, *task, placement, *acc);
+  switch (pipelink_mok_gemm_depth()) {
+    case 2: PL_STORE(2) break;
+    default: PL_STORE(4) break;
+  }
+#undef PL_STORE
 }
 #else  // PIPELINK_EMIT: host-evaluated annotations only
 #include "../include/mok_abi.h"
@@ -876,6 +1097,14 @@ PL_EXPORT(mok_gemm_fwd, mok_gemm_fwd,
           "const MokGemmTask* upcoming);");
 PL_EXPORT(mok_gemm_store, mok_gemm_store,
           "extern \"C\" __device__ void mok_gemm_store(const void* view, const MokGemmTask* task, const mok::AccFrag* acc);");
+PL_EXPORT(mok_gemm_placement, mok_gemm_placement,
+          "extern \"C\" __device__ int mok_gemm_placement(const void* view, const MokGemmTask* task);");
+PL_EXPORT(mok_gemm_fwd_small, mok_gemm_fwd_small,
+          "extern \"C\" __device__ void mok_gemm_fwd_small(const void* view, const MokGemmTask* task, "
+          "const MokCounters* counters, uint32_t* phase, mok::AccFrag* acc, const mok::GemmCarry* carry, "
+          "const MokGemmTask* upcoming);");
+PL_EXPORT(mok_gemm_store_small, mok_gemm_store_small,
+          "extern \"C\" __device__ void mok_gemm_store_small(const void* view, const MokGemmTask* task, const mok::AccFrag* acc);");
 PL_SERVE(gemm_init, "mok_gemm_init");
 PL_SERVE(gemm_fini, "mok_gemm_fini");
 PL_SERVE(gemm_stage, "mok_gemm_stage");
@@ -884,6 +1113,9 @@ PL_SERVE(gemm_wait, "mok_gemm_wait");
 PL_SERVE(gemm_prefetch, "mok_gemm_prefetch");
 PL_SERVE(gemm_fwd, "mok_gemm_fwd");
 PL_SERVE(gemm_store, "mok_gemm_store");
+PL_SERVE(gemm_placement, "mok_gemm_placement");
+PL_SERVE(gemm_fwd_small, "mok_gemm_fwd_small");
+PL_SERVE(gemm_store_small, "mok_gemm_store_small");
 // head, live for the whole kernel: the first two 16 KB buffers of the routed-row ring and of the weight
 // ring, four 1 KB buffers of weight scales, two 4 KB buffers of routed-row scales, the staged task's row tokens (1 KB)
 // and readiness counter (256 B)

@@ -102,7 +102,7 @@ typedef struct MokActResidue {
 typedef struct MokFrameworkParams {
   const int32_t* tokens_per_expert; /* [E] */
   uint32_t* workspace;              /* MOK_WS_* words + one counter per routed-row tile; all zero before a launch,
-                                       and the launch leaves them zero (except the status word) */
+                                       and the launch leaves them zero (except the status word and the poll limit) */
   int32_t num_experts;
   int32_t op;                       /* which GEMM this launch runs, or MOK_FWD_BOTH */
   int32_t num_col_tiles_gate_up;    /* column tiles of the gate/up GEMM (128 gate + 128 up columns each) */
@@ -112,8 +112,12 @@ typedef struct MokFrameworkParams {
 enum {
   MOK_WS_STATUS = 0,    /* sticky MOK_STATUS_* bits; the host reads and clears it */
   MOK_WS_FINISHED = 1,  /* workgroups that have left the launch; the last one clears the counters */
-  MOK_WS_POLL_LIMIT = 2, /* 0, or the number of polls after which a dependency wait gives up instead of the default 2^18
+  MOK_WS_POLL_LIMIT = 2, /* 0, or the number of polls after which a dependency wait gives up instead of the default 2^14
                             (for tests of the give-up path: the kernels never write it) */
+  MOK_WS_GAVE_UP = 3,   /* non-zero once a dependency wait of the running launch has given up: every later wait of that
+                            launch gives up at once; the launch's last workgroup puts it back to zero */
+  MOK_WS_QUEUE = 8,     /* eight words, one per tile list: how many of the list's tiles have been handed out beyond the two
+                            every workgroup starts with; the launch's last workgroup puts them back to zero */
   MOK_WS_COUNTERS = 32  /* first readiness counter */
 };
 

@@ -63,7 +63,50 @@ __device__ __forceinline__ int wrow0(int wave, int a) {
 }
 __device__ __forceinline__ int xrow0(int wave, int b) { return wave_x(wave) * 128 + b * 32; }
 
+// ---- tiles with little to multiply ------------------------------------------------------------------------------
+// A tile that holds at most 64 routed rows (the rows an expert has past its last full tile), or at most 64 output
+// columns per weight matrix (the columns past the last full column tile), is multiplied in another placement: every
+// wave takes 64 routed rows and up to four 32-row weight fragments, in the accumulator's fragments [a][b] with b < 2.
+//   SMALL_ROWS: all four waves share routed rows 0..63; wave w owns weight fragments a = 0 and a = 2, tile rows
+//               32 w and 128 + 32 w (for the gate/up op: 32 gate columns and the same 32 up columns).
+//   SMALL_COLS: wave w owns routed rows 64 w .. 64 w + 63; the weight fragments are tile rows 0, 32 (a = 0, 1) and,
+//               for the gate/up op, 128, 160 (a = 2, 3): 64 gate columns and the same 64 up columns.
+// Element (reg r, lane l) of fragment (a, b) is weight row wr[a] + 8 (r / 4) + 4 (l / 32) + r % 4, routed row
+// xr0 + 32 b + l % 32.  Which placement a tile has follows from its extent alone, so every owner works it out for itself.
+enum { TILE_FULL = 0, TILE_SMALL_ROWS = 1, TILE_SMALL_COLS = 2 };
+constexpr int SMALL_EXTENT = 64;
+// rows: routed rows of the tile that exist; cols: output columns (per weight matrix) from the tile's first that exist
+__device__ __forceinline__ int tile_placement(int rows, int cols) {
+  return rows <= SMALL_EXTENT ? TILE_SMALL_ROWS : cols <= SMALL_EXTENT ? TILE_SMALL_COLS : TILE_FULL;
+}
+struct SmallPlacement {
+  int xr0;    // first tile-local routed row of the wave
+  int wr[4];  // tile-local weight row of fragment a
+};
+__device__ __forceinline__ SmallPlacement small_placement(int placement, int wave) {
+  SmallPlacement p;
+  const bool rows = placement == TILE_SMALL_ROWS;
+  p.xr0 = rows ? 0 : 64 * wave;
+  p.wr[0] = rows ? 32 * wave : 0;
+  p.wr[1] = 32;
+  p.wr[2] = TILE_W / 2 + (rows ? 32 * wave : 0);
+  p.wr[3] = TILE_W / 2 + 32;
+  return p;
+}
+// the fragments a that are multiplied, as a bit mask: a = 0 and 2 for few rows; 0, 1 and (gate/up op) 2, 3 for few columns
+constexpr int SMALL_ROWS_FRAGS = 0b0101, SMALL_COLS_FRAGS_GATE_UP = 0b1111, SMALL_COLS_FRAGS_DOWN = 0b0011;
+
 typedef __attribute__((address_space(3))) void* lptr_t;
+
+// Workgroup barrier that orders the workgroup's LDS traffic and nothing else: every LDS access this wave has issued
+// has completed (lgkmcnt(0)); vector-memory operations stay in flight.  __syncthreads() also waits for every
+// outstanding global -> LDS load and every store.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
 
 // threadIdx.x as a value the compiler cannot merge with an earlier copy: code that runs after
 // a register-hungry loop derives its lane indices from this, so they are computed where they

@@ -5,6 +5,7 @@ Bars: quantiser bytes bit-exact; y within 3e-2 relative Frobenius of the oracle 
 the path's specification states for MXFP8; observed ~1.5e-3, which is bf16 output rounding);
 linked image vs one-unit control byte-identical, outputs poisoned before every launch."""
 import json
+import time
 
 import numpy as np
 import pytest
@@ -387,6 +388,19 @@ def test_a_dependency_wait_that_cannot_be_met_gives_up_and_says_so(cell):
         assert after[0] == 1                                   # MOK_STATUS_WAIT_GAVE_UP
         assert after[1] == 0 and not after[32:].any()          # the launch closed and put its counters back
         assert np.array_equal(t["hidden_q"][:, :I].cpu().numpy(), want[0])   # the gate/up tiles depend on nobody
+        # The same with the kernel's own poll limit: the first wait to give up takes 2^14 polls, every other wait of the
+        # launch then ends at once (workspace word 3, which the launch puts back to zero), so the launch is over in
+        # tens of milliseconds however many tiles wait.
+        ws[2] = 0
+        t["workspace"].copy_(ws)
+        be.synchronize()
+        t0 = time.perf_counter()
+        s.launch()
+        be.synchronize()
+        elapsed = time.perf_counter() - t0
+        after = t["workspace"].cpu()
+        assert after[0] == 1 and after[3] == 0 and not after[32:].any()
+        assert elapsed < 0.1, f"a launch whose waits cannot be met took {elapsed * 1e3:.0f} ms"
         t["workspace"].zero_()                                 # the host clears the status (and the poll limit)
         t["y"].fill_(float("nan"))
         s.launch()

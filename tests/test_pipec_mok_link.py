@@ -41,7 +41,9 @@ def test_link_json_records_the_solved_cell(cell):
     assert [e["stage_id"] for e in link["params"]["entries"]] == ["mok.framework", "mok.gemm", "mok.act"]
     assert link["params"]["total_bytes"] == 32 + 264 + 40
     assert {e["channel"] for e in link["protocol_expansions"]} == {"gemm_init", "gemm_fini", "gemm_stage", "gemm_ready", "gemm_wait", "gemm_prefetch",
-                                                                   "gemm_fwd", "gemm_store", "act_init", "act_fwd"}
+                                                                   "gemm_fwd", "gemm_store", "act_init", "act_fwd",
+                                                                   # tiles of few rows / few columns: their own exports
+                                                                   "gemm_placement", "gemm_fwd_small", "gemm_store_small", "act_fwd_small"}
     obs = link["observed"]
     assert obs["calls"] == 0 and obs["private_segment_fixed_size"] <= 64 and obs["mfma"] >= 16   # a few dwords spilled in the tile set-up at most
     assert obs["vgpr_count"] <= link["regs_cap"] == 512
