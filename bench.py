@@ -56,17 +56,25 @@ def traffic_bytes():
 
 
 def executed_flops(counts):
-    """Flops the kernel's waves execute for these per-expert row counts: a wave multiplies its 128 x 128 share of a
-    tile over the whole contraction unless the share starts past the expert's last row or past the last output
-    column (then it only loads).  Shares that are partly past the end are multiplied in full."""
+    """Flops the kernel's waves execute for these per-expert row counts.  A full tile: a wave multiplies its 128 x 128
+    share over the whole contraction unless the share starts past the expert's last row or past the last output
+    column (then it only loads); shares that are partly past the end are multiplied in full.  A tile of at most 64
+    rows or at most 64 columns (per matrix) is in the small placement: four waves x 64 rows x the 32-row weight
+    fragments they hold (few rows: 2 per wave; few columns: 2 per wave and matrix)."""
     total = 0.0
     for c in counts:
         for first in range(0, int(c), TILE):
-            row_waves = 1 if int(c) - first <= TILE // 2 else 2
-            for cols, k, step in ((I, H, TILE // 2), (H, I, TILE)):  # gate/up (per matrix), down
+            rows = int(c) - first
+            row_waves = 1 if rows <= TILE // 2 else 2
+            for cols, k, step, matrices in ((I, H, TILE // 2, 2), (H, I, TILE, 1)):  # gate/up (two matrices), down
                 for col_begin in range(0, cols, step):
-                    col_waves = sum(col_begin + w * 64 < cols for w in (0, 1))
-                    total += row_waves * col_waves * 128 * 128 * 2.0 * k
+                    if rows <= 64:      # few rows: every wave 64 rows x 2 fragments of 32 weight rows
+                        total += 4 * 64 * 64 * 2.0 * k
+                    elif cols - col_begin <= 64:  # few columns: every wave 64 rows x 64 columns of each matrix
+                        total += 4 * 64 * 64 * matrices * 2.0 * k
+                    else:
+                        col_waves = sum(col_begin + w * 64 < cols for w in (0, 1))
+                        total += row_waves * col_waves * 128 * 128 * 2.0 * k  # (gate/up: 64 gate + 64 up columns per wave)
     return total
 
 
@@ -209,8 +217,8 @@ def mfma_ceiling(be, torch, seconds=1.0):
 
 
 def cpu_baseline(inp, row_major, slice_tokens=1024):
-    """The oracle on the host cores: the whole batch of the same inputs (one run after one warm-up), and its first
-    `slice_tokens` tokens (median of 3 after a warm-up)."""
+    """The oracle on the host cores: the whole batch of the same inputs, and its first `slice_tokens` tokens (each the
+    median of 3 runs after a warm-up)."""
     import torch
     from oracle import moe_ffn
     from pipelink_amd.host import mok_inputs
@@ -236,10 +244,10 @@ def cpu_baseline(inp, row_major, slice_tokens=1024):
         return statistics.median(times)
 
     sec_slice = timed(slice_tokens, 3)
-    sec_full = timed(T, 1)
+    sec_full = timed(T, 3)
     return {"value": round(FLOPS_TOTAL / sec_full / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
             "sample": f"the whole batch ({T} tokens, {T * TOPK} routed rows; all {E} experts' weights dequantised inside the "
-                      f"timed region): one run after 1 warm-up, {sec_full * 1e3:.0f} ms per forward, torch {torch.__version__} fp32",
+                      f"timed region): median of 3 runs after 1 warm-up, {sec_full * 1e3:.0f} ms per forward, torch {torch.__version__} fp32",
             "slice": {"value": round(FLOPS_TOTAL * slice_tokens / T / sec_slice / 1e12, 4), "tokens": slice_tokens,
                       "ms_per_forward": round(sec_slice * 1e3), "runs": "median of 3 after 1 warm-up"}}
 

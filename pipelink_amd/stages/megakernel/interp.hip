@@ -98,7 +98,11 @@ __device__ __forceinline__ bool poll(uint32_t* word, uint32_t target, bool local
 }
 // first half of barrier number `generation` (1, 2, ...) of the launch: this workgroup has finished what comes before it
 __device__ __forceinline__ void grid_arrive(const MkModel& m, uint32_t generation) {
-  __syncthreads();  // every wave's stores have been issued and acknowledged by the L2
+  // Every wave first waits until its own stores have been written through (a store leaves the wave's vector-memory
+  // count when it is acknowledged; the barrier's workgroup-scope fence does not wait for that): what the workgroup hands
+  // the others is in memory before it says that it has arrived.
+  __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+  __syncthreads();
   if (threadIdx.x == 0) {
     const uint32_t xcd = blockIdx.x % NUM_XCD;
     const uint32_t members = (gridDim.x - xcd + NUM_XCD - 1) / NUM_XCD;
@@ -107,9 +111,11 @@ __device__ __forceinline__ void grid_arrive(const MkModel& m, uint32_t generatio
       __hip_atomic_fetch_add(m.sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
-// second half: every workgroup has arrived at barrier number pending->barrier.  After a give-up a workgroup waits for
-// no barrier of the launch any more: the step's results are void by then, and the launch should end quickly.  (The others waiting at that barrier give up within the same
-// period; a workgroup that was not running finds every barrier complete when it gets there, because arrivals go on.)
+// second half: every workgroup has arrived at barrier number pending->barrier.  The wait is bounded by SPIN_LIMIT polls
+// and nothing else: a workgroup that has given up one barrier polls the next one again for as long (keeping "gave up
+// once" across the ops was measured and costs more than it saves, see SPIN_LIMIT), so a launch that cannot complete
+// pays up to SPIN_LIMIT polls per barrier and workgroup.  (A workgroup that was not running finds every barrier
+// complete when it gets there, because arrivals go on.)
 __device__ __forceinline__ void grid_wait(const MkModel& m, MkPending* pending) {
   const uint32_t generation = pending->barrier;
   if (threadIdx.x == 0) {

@@ -70,6 +70,63 @@ def test_static_entry_point_matches_forward_on_two_calls_in_a_row():
             assert not torch.isnan(out["y"].float()).any()
 
 
+def test_static_entry_point_allocates_nothing_and_can_be_captured():
+    """What the entry point is for: the device's free memory is the same after the calls as before them (no hipMalloc /
+    hipFree, by the library or by torch), and two calls in a row are captured into a HIP graph on a fresh stream -- a
+    new problem each, where plk_mok_forward would have to upload an image and says PLK_E_CONTRACT -- and every replay
+    writes the bytes of the eager forward."""
+    from pipelink_amd.host import mok_inputs
+    from pipelink_amd.host.backend import HipBackend, PlkError
+    from pipelink_amd.host.mok import MoKSession
+    from pipelink_amd.stages.mok import build as mok_build
+
+    paths = mok_build.images()
+    link = json.loads(paths["link_json"].read_text())
+    shapes = [(520, 320, 384, 4, 2, 31, 384), (96, 256, 320, 8, 2, 32, None)]
+    with MoKSession(paths["linked"].read_bytes(), link) as sess, MoKSession(paths["linked"].read_bytes(), link) as fresh:
+        cases = [_device_problem(sess, mok_inputs.generate(T, H, I, E, k, seed=seed), H, I, pitch) for T, H, I, E, k, seed, pitch in shapes]
+        expected = []
+        for prob, out, _ in cases:
+            _poison(out)
+            sess.forward(prob)
+            expected.append(_snapshot(out))
+        for prob, out, _ in cases:
+            _poison(out)
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        for prob, out, _ in cases:
+            sess.forward_static(prob)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        for (prob, out, _), want in zip(cases, expected):
+            assert all(torch.equal(g, w) for g, w in zip(_snapshot(out), want))
+
+        be = HipBackend(0, 0)
+        stream = be.stream_create()
+        # a session that has never seen these problems: plk_mok_forward would have to upload their params images
+        with pytest.raises(PlkError):
+            be.capture(stream, lambda: fresh.forward(cases[0][0], stream=stream))
+
+        def body():
+            for prob, out, _ in cases:
+                fresh.forward_static(prob, stream=stream)
+
+        graph = be.capture(stream, body)
+        try:
+            for replay in range(3):
+                for prob, out, _ in cases:
+                    _poison(out)
+                torch.cuda.synchronize()   # the program's own eager work and synchronisation between the replays
+                graph.launch(stream)
+                be.synchronize(stream)
+                for (prob, out, _), want in zip(cases, expected):
+                    assert all(torch.equal(g, w) for g, w in zip(_snapshot(out), want)), f"replay {replay}"
+            assert fresh.status() == 0
+        finally:
+            graph.close()
+            be.close()
+
+
 def test_static_entry_point_rejects_sizes_beyond_its_area():
     from ctypes import sizeof
 
