@@ -216,6 +216,20 @@ __device__ __forceinline__ v8i read_frag(const unsigned char* slot, int off) {
   return r;
 }
 
+// A zeroed accumulator fragment.  Written by one instruction of the matrix pipe (an integer MFMA of zeros, eight
+// passes) instead of sixteen register writes: a wave issues in order, one instruction every four or five clocks, and 256
+// writes per tile are half a microsecond in which it issues nothing else.  (The zero is opaque to the compiler, which
+// would otherwise fold the product back into the writes.)
+// The instruction is written out so that its result is born in the accumulator registers (left to the compiler it
+// may be born in vector registers and copied, which the mainloop has none to spare for); nothing reads the fragment
+// for hundreds of instructions, so the matrix pipe's result latency needs no attention here.
+__device__ __forceinline__ v16f zero_fragment() {
+  long z = 0;
+  v16f f;
+  asm volatile("v_mfma_i32_32x32x16_i8 %0, %1, %1, 0" : "=a"(f) : "v"(z));
+  return f;
+}
+
 // Workgroup barrier without the release/acquire fence of __syncthreads(): a fence would
 // drain every outstanding global->LDS load (vmcnt(0)) and serialise the ring.  Ordering of
 // the LDS traffic is by the explicit s_waitcnt in front of it.
@@ -374,7 +388,8 @@ __device__ __forceinline__ Views views_of(const MokGemmResidue& g, const MokGemm
 
 // The gathered part of a tile's loader: routed row -> source row goes through row_token for the gate/up op, a
 // dependent load, which `stage` has taken ahead: the tokens are read from LDS (those of rows past the end are zero there).
-__device__ __forceinline__ void gather_rows(const MokGemmResidue& g, const Views& v, const MokGemmTask& t, GemmCarry& c) {
+// (`few`: a tile of at most 64 rows in the deep ring below, whose wave w loads routed rows 16 w .. 16 w + 15: xsrc[0] only.)
+__device__ __forceinline__ void gather_rows(const MokGemmResidue& g, const Views& v, const MokGemmTask& t, GemmCarry& c, bool few = false) {
   const int tid = fresh_tid();
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -386,7 +401,7 @@ __device__ __forceinline__ void gather_rows(const MokGemmResidue& g, const Views
   const int chunk = 16 * ((lane & 3) ^ swizzle(lrow));
 #pragma unroll
   for (int i = 0; i < X_GROUPS; ++i) {
-    const int trow = (wave * X_GROUPS + i) * 16 + lrow;  // tile-local routed row
+    const int trow = few ? wave * 16 + lrow : (wave * X_GROUPS + i) * 16 + lrow;  // tile-local routed row
     const int row = t.row_begin + trow;
     const int safe = row < t.row_end ? row : t.row_end - 1;
     const int src = gathered ? staged_token[trow] : safe;
@@ -488,13 +503,85 @@ __device__ __forceinline__ int loads_younger_than_slot(int slot, int last, int n
   return younger;
 }
 
+
+// ---- tiles of at most 64 routed rows: a deeper ring ---------------------------------------------------------------
+// Such a tile has a quarter of a full tile's MFMAs and as many steps: it takes as long as its loads take to arrive,
+// and a load that is in flight for three steps' time (the full tile's ring) bounds a step from below by a third of
+// the latency of a load.  Its routed rows need 4 KB per slot, not 16: the same LDS holds seven slots of 16 KB of
+// weight rows + 4 KB of routed rows, the first three in the head (where the tile before leaves room while its
+// epilogue uses the arena), four in the arena.  Wave w loads its 64 weight rows as in the full tile and routed rows
+// 16 w .. 16 w + 15; one slot per step, all of it at once (five loads a wave).  Scale buffers and their loads are the
+// full tile's.  Needs the arena of ring depth 4.
+constexpr int FEW_DEPTH = 7;
+constexpr int FEW_HEAD_SLOTS = 3;
+constexpr int FEW_X_BYTES = SMALL_EXTENT * K_SLOT;        // 4 KB
+constexpr int FEW_SLOT_BYTES = BUF_BYTES + FEW_X_BYTES;   // weight rows, then routed rows
+constexpr int FEW_LOADS = W_LOADS + 1;                    // tile loads of one slot, per wave
+static_assert(FEW_HEAD_SLOTS * FEW_SLOT_BYTES <= 4 * BUF_BYTES, "the first slots fit where the full tile's first buffers are");
+struct FewRing {
+  unsigned char* head;
+  unsigned char* arena;
+  __device__ __forceinline__ FewRing() : head(pipelink_smem + pipelink_mok_gemm_head()), arena(pipelink_smem + pipelink_mok_gemm_arena()) {}
+  __device__ __forceinline__ unsigned char* slot(int pos) const {  // pos = slot number mod FEW_DEPTH
+    return pos < FEW_HEAD_SLOTS ? head + pos * FEW_SLOT_BYTES : arena + (pos - FEW_HEAD_SLOTS) * FEW_SLOT_BYTES;
+  }
+};
+// all loads of slot s, into ring position pos: [scale loads] [routed rows] [weight rows]
+__device__ __forceinline__ void issue_few(const Loader& ld, const FewRing& ring, const Rings<4>& r, int s, int pos, int n) {
+  if (s >= n) return;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t kbyte = (uint32_t)s * K_SLOT;
+  const int j8 = s & 7;
+  if (j8 == 0) buf16_to_lds_device_scope(ld.xsc, ld.xscsrc, kbyte >> 5, r.xscale() + ((s >> 3) & 1) * (TILE_X * 16) + wave * 1024);
+  if ((j8 & 1) == 0) buf4_to_lds(ld.wsc, ld.wscsrc, (uint32_t)(s >> 1) * ld.wsc_pair_pitch, r.wscale() + (j8 >> 1) * (TILE_W * 4) + wave * 256);
+  unsigned char* base = ring.slot(pos);
+  buf16_to_lds(ld.x, ld.xsrc[0], kbyte, base + BUF_BYTES + wave * 1024);
+  const uint32_t wslot = (uint32_t)s * ld.w_slot_pitch;
+#pragma unroll
+  for (int i = 0; i < W_GROUPS; ++i) buf16_to_lds(ld.w, ld.wsrc[i], wslot, base + ld.dst + i * 1024);
+}
+// tile loads that may still be outstanding when slot `slot` is needed and steps up to `last` have been issued (step u
+// issues slot u + FEW_DEPTH)
+__device__ __forceinline__ int few_younger(int slot, int last, int n) {
+  int younger = 0;
+  for (int u = slot + 1 - FEW_DEPTH; u <= last; ++u) younger += u + FEW_DEPTH < n ? FEW_LOADS : 0;
+  return younger;
+}
+__device__ __forceinline__ void wait_few(int loads) {  // a multiple of FEW_LOADS, at most (FEW_DEPTH - 1) of them
+  switch (__builtin_amdgcn_readfirstlane(loads) / FEW_LOADS) {
+    case 0: wait_loads_and_reads<0>(); break;
+    case 1: wait_loads_and_reads<FEW_LOADS>(); break;
+    case 2: wait_loads_and_reads<2 * FEW_LOADS>(); break;
+    case 3: wait_loads_and_reads<3 * FEW_LOADS>(); break;
+    case 4: wait_loads_and_reads<4 * FEW_LOADS>(); break;
+    case 5: wait_loads_and_reads<5 * FEW_LOADS>(); break;
+    default: wait_loads_and_reads<6 * FEW_LOADS>(); break;
+  }
+}
+// which placement the task's tile has: its routed rows that exist, its output columns that exist
+__device__ __forceinline__ int placement_of(const MokGemmResidue& g, const MokGemmTask& t) {
+  const int cols = (t.op == MOK_GEMM_FWD_ROUTED_GATE_UP ? g.w_gate.rows : g.w_down.rows) - t.col_begin;
+  return tile_placement(t.row_end - t.row_begin, cols);
+}
+
 template <int DEPTH>
 __device__ __forceinline__ void prefetch(const MokGemmResidue& g, const MokGemmTask& t, GemmCarry& c) {
   const Views v = views_of(g, t);
+  const int n = v.act.k / K_SLOT;
+  if constexpr (DEPTH >= 4) {
+    if (placement_of(g, t) == TILE_SMALL_ROWS) {  // the deep ring's first slots
+      gather_rows(g, v, t, c, true);
+      const Loader ld = make_loader(v, t, c);
+      const FewRing ring;
+      const Rings<4> r;
+#pragma unroll
+      for (int s = 0; s < FEW_HEAD_SLOTS; ++s) issue_few(ld, ring, r, s, s, n);
+      return;
+    }
+  }
   gather_rows(g, v, t, c);
   const Loader ld = make_loader(v, t, c);
   const Rings<DEPTH> r;
-  const int n = v.act.k / K_SLOT;
   issue_step(ld, r, -DEPTH, n, 0, 1, 0);
   issue_step(ld, r, 1 - DEPTH, n, 0, 1, 1);
 }
@@ -528,14 +615,14 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
     wscoff[a] = wl * 4;
   }
 
-  // cleared for an idle wave as well: an accumulator it left unwritten would be the previous
-  // tile's, kept alive across the loop
+  // The accumulator is cleared further down, on each of the two paths by itself (an idle wave's as well: one it left
+  // unwritten would be the previous tile's, kept alive across the loop).
+  auto clear_accumulator = [&]() {
 #pragma unroll
-  for (int a = 0; a < WFRAGS; ++a)
+    for (int a = 0; a < WFRAGS; ++a)
 #pragma unroll
-    for (int b = 0; b < XFRAGS; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc.v[a][b][r] = 0.0f;
+      for (int b = 0; b < XFRAGS; ++b) acc.v[a][b] = zero_fragment();
+  };
 
   static_assert(DEPTH % 2 == 0, "routed-row pairs start on even steps");
   // steady state, every step issuing: what may be outstanding when step t waits for slot t+1
@@ -575,9 +662,11 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
       step(j + 1);
     }
     wg_barrier();
+    clear_accumulator();
     return;
   }
 
+  clear_accumulator();
   Operands even, odd;
   int sx[XFRAGS], sw[WFRAGS], sxn[XFRAGS], swn[WFRAGS];
   read_operands(even, r.x(0), r.w(0), xoff, woff);
@@ -754,10 +843,7 @@ __device__ __forceinline__ void mainloop_small(const MokGemmResidue& g, const Mo
   for (int a = 0; a < 4; ++a)
 #pragma unroll
     for (int b = 0; b < 2; ++b)
-      if (used(a)) {
-#pragma unroll
-        for (int q = 0; q < 16; ++q) acc.v[a][b][q] = 0.0f;
-      }
+      if (used(a)) acc.v[a][b] = zero_fragment();
 
   // the prologue of the full tile: steps -DEPTH and 1 - DEPTH were issued by `prefetch`
 #pragma unroll
@@ -830,10 +916,102 @@ __device__ __forceinline__ void mainloop_small(const MokGemmResidue& g, const Mo
   wg_barrier();  // every wave holds its last operands in registers: the ring is free
 }
 
-// which placement the task's tile has: its routed rows that exist, its output columns that exist
-__device__ __forceinline__ int placement_of(const MokGemmResidue& g, const MokGemmTask& t) {
-  const int cols = (t.op == MOK_GEMM_FWD_ROUTED_GATE_UP ? g.w_gate.rows : g.w_down.rows) - t.col_begin;
-  return tile_placement(t.row_end - t.row_begin, cols);
+
+
+// The mainloop of a tile of at most 64 rows in the deep ring (ring depth 4 and up; mainloop_small<DEPTH, SMALL_ROWS_FRAGS>
+// otherwise): the small placement's fragments a = 0 and a = 2, two routed-row fragments, four MFMAs a step.
+__device__ __forceinline__ void mainloop_few_rows(const MokGemmResidue& g, const MokGemmTask& t, AccFrag& acc, const GemmCarry& carry,
+                                                  const MokGemmTask* upcoming, const MokCounters& counters) {
+  const int tid = fresh_tid();  // nothing of this path is to be computed ahead and kept across full tiles
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r32 = lane & 31;
+  const int half = lane >> 5;
+  const Views v = views_of(g, t);
+  const int n = v.act.k / K_SLOT;
+  const FewRing ring;
+  const Rings<4> r;
+  const Loader ld = make_loader(v, t, carry);
+  const SmallPlacement sp = small_placement(TILE_SMALL_ROWS, wave);
+  int xoff[2], xscoff[2], woff[2], wscoff[2];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const int row = 32 * b + r32;
+    xoff[b] = BUF_BYTES + row * K_SLOT + 16 * (half ^ swizzle(row));
+    xscoff[b] = row * 16;
+  }
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    const int wl = sp.wr[2 * a] + r32;
+    woff[a] = wl * K_SLOT + 16 * (half ^ swizzle(wl));
+    wscoff[a] = wl * 4;
+  }
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) acc.v[2 * a][b] = zero_fragment();
+
+  // slots 0 .. FEW_HEAD_SLOTS - 1 were asked for by `prefetch`; the rest of the ring now
+#pragma unroll
+  for (int s = FEW_HEAD_SLOTS; s < FEW_DEPTH; ++s) issue_few(ld, ring, r, s, s, n);
+  if (upcoming->op != 0) stage(g, *upcoming, counters);
+  wait_few(few_younger(0, -1, n));
+  wg_barrier();
+
+  struct FewOperands {
+    v8i x[2], w[2];
+  } even, odd;
+  int sx[2], sw[2], sxn[2], swn[2];
+  auto read_operands_few = [&](FewOperands& o, const unsigned char* slot) {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) o.x[b] = read_frag(slot, xoff[b]);
+#pragma unroll
+    for (int a = 0; a < 2; ++a) o.w[a] = read_frag(slot, woff[a]);
+  };
+  auto read_scales_few = [&](int (&sx_)[2], int (&sw_)[2], int j) {  // of the pair of slots that starts at slot j (j even)
+    const int c = (j & 7) >> 1;
+    const unsigned char* xbuf = r.xscale() + ((j >> 3) & 1) * (TILE_X * 16);
+    const unsigned char* wbuf = r.wscale() + c * (TILE_W * 4);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) sx_[b] = (int)(*reinterpret_cast<const uint32_t*>(xbuf + 4 * c + xscoff[b]) >> (8 * half));
+#pragma unroll
+    for (int a = 0; a < 2; ++a) sw_[a] = (int)(*reinterpret_cast<const uint32_t*>(wbuf + wscoff[a]) >> (8 * half));
+  };
+  auto multiply = [&](auto ODD_, const FewOperands& o) {
+    constexpr bool ODD = decltype(ODD_)::value;
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+        acc.v[2 * a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.w[a], o.x[b], acc.v[2 * a][b], 0, 0, ODD ? 2 : 0, sw[a],
+                                                                          ODD ? 2 : 0, sx[b]);
+  };
+  read_operands_few(even, ring.slot(0));
+  read_scales_few(sx, sw, 0);
+  int pos = 0;  // ring position of slot t_ in `advance`
+  // step t_: slot t_ + 1 has landed for every wave and every wave holds slot t_ in registers, whose place takes slot
+  // t_ + FEW_DEPTH
+  auto advance = [&](int t_, FewOperands& next) {
+    wait_few(few_younger(t_ + 1, t_ - 1, n));
+    wg_barrier();
+    issue_few(ld, ring, r, t_ + FEW_DEPTH, pos, n);
+    pos = pos + 1 == FEW_DEPTH ? 0 : pos + 1;
+    read_operands_few(next, ring.slot(pos));
+  };
+  int j = 0;
+  for (; j + 1 < n; j += 2) {
+    advance(j, odd);
+    multiply(std::false_type{}, even);
+    advance(j + 1, even);
+    read_scales_few(sxn, swn, j + 2);
+    multiply(std::true_type{}, odd);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) sx[b] = sxn[b];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) sw[a] = swn[a];
+  }
+  if (n & 1) multiply(std::false_type{}, even);
+  wg_barrier();  // every wave holds its last operands in registers: the ring is free
 }
 
 // bf16 epilogue of the down op.  The accumulator is transposed through the arena buffers (idle
@@ -1044,7 +1222,11 @@ extern "C" __device__ void mok_gemm_fwd_small(const void* view, const MokGemmTas
       switch (frags) { PL_SMALL(2, mok::SMALL_ROWS_FRAGS) PL_SMALL(2, mok::SMALL_COLS_FRAGS_GATE_UP) PL_SMALL(2, mok::SMALL_COLS_FRAGS_DOWN) }
       break;
     default:
-      switch (frags) { PL_SMALL(4, mok::SMALL_ROWS_FRAGS) PL_SMALL(4, mok::SMALL_COLS_FRAGS_GATE_UP) PL_SMALL(4, mok::SMALL_COLS_FRAGS_DOWN) }
+      if (placement == mok::TILE_SMALL_ROWS) {  // (the deep ring needs the arena of depth 4; mok_gemm_prefetch decides alike)
+        mok_gemm_owner::mainloop_few_rows(g, *task, *acc, *carry, upcoming, *counters);
+        break;
+      }
+      switch (frags) { PL_SMALL(4, mok::SMALL_COLS_FRAGS_GATE_UP) PL_SMALL(4, mok::SMALL_COLS_FRAGS_DOWN) }
       break;
   }
 #undef PL_SMALL
