@@ -478,21 +478,21 @@ __device__ __forceinline__ void issue_step(const Loader& ld, const Rings<DEPTH>&
 }
 // tile loads issue_step(u) issues: routed rows, weight rows
 template <int DEPTH>
-__device__ __forceinline__ int x_loads_in(int u, int n) {
+__device__ __forceinline__ constexpr int x_loads_in(int u, int n) {
   const int s = u + DEPTH;
   const int pair = (u & 1) ? s - 1 : s;
   if (pair >= n) return 0;
   return DEPTH >= 4 ? X_LOADS / 2 : ((u & 1) == 0 ? X_LOADS : 0);
 }
 template <int DEPTH>
-__device__ __forceinline__ int w_loads_in(int u, int n) { return u + DEPTH < n ? W_LOADS : 0; }
+__device__ __forceinline__ constexpr int w_loads_in(int u, int n) { return u + DEPTH < n ? W_LOADS : 0; }
 // Tile loads that may still be outstanding when slot `slot` is needed and steps up to `last`
 // have been issued (step t waits for slot t+1 with last = t-1; the prologue waits for slot 0
 // with last = -1).  The slot's weight rows are the last loads of step slot-DEPTH; its routed
 // rows come no later, except that with split pairs groups 2-3 of an even slot are issued at
 // the start of step slot+1-DEPTH.
 template <int DEPTH>
-__device__ __forceinline__ int loads_younger_than_slot(int slot, int last, int n) {
+__device__ __forceinline__ constexpr int loads_younger_than_slot(int slot, int last, int n) {
   int younger = 0;
   int first = slot + 1 - DEPTH;  // first step all of whose loads are younger
   if (DEPTH >= 4 && (slot & 1) == 0) {
@@ -636,7 +636,11 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   // behind the slot they need, and loads return in order, so one or two more of the youngest only make the next few
   // waits ask for as many more of the oldest.
   if (upcoming->op != 0) stage(g, *upcoming, counters);
-  wait_loads_and_reads_dyn(loads_younger_than_slot<DEPTH>(0, -1, n));
+  // (with at least DEPTH slots every step up to here has issued its loads: the count is a constant then, and the wait
+  // one instruction instead of a computation and a branch table)
+  constexpr int ALL_ISSUED = loads_younger_than_slot<DEPTH>(0, -1, 1 << 20);
+  if (n >= DEPTH) wait_loads_and_reads<ALL_ISSUED>();
+  else wait_loads_and_reads_dyn(loads_younger_than_slot<DEPTH>(0, -1, n));
   wg_barrier();
   auto xnext = [](int b, int by) {  // (b + by) mod XDEPTH for 0 <= b < XDEPTH, 0 <= by <= XDEPTH
     const int c = b + by;
@@ -849,7 +853,11 @@ __device__ __forceinline__ void mainloop_small(const MokGemmResidue& g, const Mo
 #pragma unroll
   for (int u = 2 - DEPTH; u < 0; ++u) issue_step(ld, r, u, n, (u + DEPTH) & ~1, ((u + DEPTH) & ~1) + 1, u + DEPTH);
   if (upcoming->op != 0) stage(g, *upcoming, counters);
-  wait_loads_and_reads_dyn(loads_younger_than_slot<DEPTH>(0, -1, n));
+  // (with at least DEPTH slots every step up to here has issued its loads: the count is a constant then, and the wait
+  // one instruction instead of a computation and a branch table)
+  constexpr int ALL_ISSUED = loads_younger_than_slot<DEPTH>(0, -1, 1 << 20);
+  if (n >= DEPTH) wait_loads_and_reads<ALL_ISSUED>();
+  else wait_loads_and_reads_dyn(loads_younger_than_slot<DEPTH>(0, -1, n));
   wg_barrier();
 
   auto xnext = [](int b, int by) {
