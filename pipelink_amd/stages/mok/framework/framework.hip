@@ -10,14 +10,16 @@
 // One launch runs both GEMMs (op MOK_FWD_BOTH) or one of them.  The tiles are in eight lists, one per XCD (workgroup
 // id % 8): list q holds the tiles of an eighth of the routed-row tiles -- the gate/up tiles first, then the down tiles
 // of the same rows; within each, expert by expert, column tile by column tile, row tiles innermost, so that
-// workgroups that run at the same time share a weight tile and one XCD's L2 sees a contiguous run of experts.  The
-// schedule is static: the workgroups of an XCD take the items of its list in turn (the reference asks the cluster
-// launch control for its next tile, interp_fwd.cu:137-160; tiles of one size gain nothing from that here, and a
-// static turn costs no atomic and no barrier).  A down tile reads rows of `hidden` that up to 23 other workgroups
-// write: it waits until the row tile's readiness counter (MokCounters) has reached the number of gate/up column
-// tiles.  Every workgroup runs all its gate/up tiles before its first down tile, gate/up tiles wait for nothing, and
-// a workgroup only ever waits while it holds no unfinished tile: so the tiles a wait depends on are finished or
-// running, no wait can last, and each is bounded anyway.
+// workgroups that run at the same time share a weight tile and one XCD's L2 sees a contiguous run of experts.  A
+// workgroup's first two tiles are fixed by its id; after that the list's queue (a word of the workspace) hands the
+// tiles out in list order, one atomic per tile, and a workgroup whose list is handed out asks the next list's queue
+// (the reference asks the cluster launch control for its next tile, interp_fwd.cu:137-160).  Tiles differ in cost
+// (full ones, and those of few rows or few columns, which have a placement of their own), and turns of equal length
+// leave the workgroups that drew the full ones tiles behind the others.  A down tile reads rows of `hidden` that up
+// to 23 other workgroups write: it waits until the row tile's readiness counter (MokCounters) has reached the number
+// of gate/up column tiles.  In every list all gate/up tiles come before the first down tile and the queue hands out
+// in that order, gate/up tiles wait for nothing, and a workgroup only ever waits while it holds no unfinished tile:
+// so the tiles a wait depends on are finished or running, no wait can last, and each is bounded anyway.
 //
 // Per workgroup the tiles are software-pipelined: the next tile's row tokens and readiness counter are requested
 // behind the current tile's first loads (mok_gemm_fwd's `upcoming`), and its first loads are issued between the
