@@ -27,6 +27,7 @@
 #include <pipelink/stage.hpp>
 #ifndef PIPELINK_EMIT
 #include "../include/mok_device.hpp"
+#include "schedule.hpp"
 
 extern "C" __device__ int pipelink_mok_fw_sched();  // byte offset of the schedule table in dynamic LDS
 
@@ -53,65 +54,7 @@ extern "C" __device__ void pipelink_call_act_fwd_small(const void* view, const M
 extern __shared__ __attribute__((aligned(1024))) unsigned char pipelink_smem[];
 
 namespace mok_framework {
-constexpr int MAX_EXPERTS = 256;
-constexpr int NUM_XCD = 8;       // lists
-
-// the schedule's tables in LDS: exclusive prefix sums per expert, and one word of the last workgroup
-struct Tables {
-  int row_begin[MAX_EXPERTS + 1];
-  int tile_begin[MAX_EXPERTS + 1];
-  uint32_t last;   // 1 in the workgroup that leaves the launch last
-  uint32_t claim;  // what the list's queue answered this workgroup's last request
-};
-
-struct Schedule {
-  const MokFrameworkParams& g;
-  const Tables& tab;
-  int row_tiles;  // of all experts
-  int gate_up_cols, down_cols;  // column tiles of the GEMMs this launch runs (0: not run)
-
-  // List q: the q-th eighth of the gate/up tiles (all experts' tiles in one sequence: expert by expert, column tile by
-  // column tile, row tiles innermost), then the q-th eighth of the down tiles.
-  __device__ __forceinline__ int share(int q, int total) const { return (int)((long long)q * total / NUM_XCD); }
-  __device__ __forceinline__ int length(int q) const {
-    const int gu = row_tiles * gate_up_cols, d = row_tiles * down_cols;
-    return share(q + 1, gu) - share(q, gu) + share(q + 1, d) - share(q, d);
-  }
-
-  // item i of list q -> task.  `cursor` is the expert of the item this workgroup decoded last: a workgroup's items
-  // come in growing order as long as it stays in one GEMM, so the search usually ends where it starts.
-  __device__ __forceinline__ MokGemmTask decode(int q, int i, int& cursor) const {
-    const int gu = row_tiles * gate_up_cols, d = row_tiles * down_cols;
-    const int gate_up_items = share(q + 1, gu) - share(q, gu);
-    const bool gate_up = i < gate_up_items;
-    const int idx = gate_up ? share(q, gu) + i : share(q, d) + i - gate_up_items;  // in the sequence of its GEMM's tiles
-    const int cols = gate_up ? gate_up_cols : down_cols;
-    // last e with tile_begin[e] * cols <= idx: it has row tiles, since tile_begin[e + 1] * cols > idx
-    int lo = cursor;
-    if (tab.tile_begin[lo] * cols > idx) lo = 0;  // the other GEMM: from the start
-    while (lo + 1 < g.num_experts && tab.tile_begin[lo + 1] * cols <= idx) ++lo;
-    cursor = lo;
-    const int e = __builtin_amdgcn_readfirstlane(lo);
-    const int t0 = tab.tile_begin[e], t1 = tab.tile_begin[e + 1];
-    const int local = idx - t0 * cols;
-    const int col = local / (t1 - t0);
-    const int tile = t0 + local - col * (t1 - t0);  // row tile, counted over all experts
-    const int first = tab.row_begin[e] + (tile - tab.tile_begin[e]) * mok::TILE_X;
-    const bool both = g.op == MOK_FWD_BOTH;
-    // wave-uniform by construction; say so, so that the task lives in scalar registers
-    MokGemmTask t;
-    t.op = gate_up ? MOK_GEMM_FWD_ROUTED_GATE_UP : MOK_GEMM_FWD_ROUTED_DOWN;
-    t.expert = e;
-    t.row_begin = __builtin_amdgcn_readfirstlane(first);
-    t.row_end = __builtin_amdgcn_readfirstlane(tab.row_begin[e + 1]);
-    t.col_begin = __builtin_amdgcn_readfirstlane(col * (gate_up ? mok::TILE_W / 2 : mok::TILE_W));
-    t.task_idx = __builtin_amdgcn_readfirstlane(q << 24 | i);
-    t.counter_idx = __builtin_amdgcn_readfirstlane(both ? tile : -1);
-    t.wait_target = gate_up ? 0 : gate_up_cols;
-    t.flags = 0u;
-    return t;
-  }
-};
+static_assert(TILE_X == mok::TILE_X && TILE_W == mok::TILE_W, "the schedule's tile is the GEMM owner's");
 
 // A tile with little to multiply (mok::tile_placement): mainloop, the next tile's first loads, epilogue -- what the
 // worker's loop does for a full tile, through the owners' exports for the small placement, and in a function of its
@@ -173,18 +116,7 @@ extern "C" __device__ void mok_framework_worker(const void* params, unsigned var
   pipelink_call_act_init(&view);
 
   // exclusive prefix sums of rows and row tiles per expert (every workgroup computes its own copy)
-  if (threadIdx.x == 0) {
-    int rows = 0, tiles = 0;
-    for (int e = 0; e < ne; ++e) {
-      tab.row_begin[e] = rows;
-      tab.tile_begin[e] = tiles;
-      const int c = g.tokens_per_expert[e];
-      rows += c;
-      tiles += (c + mok::TILE_X - 1) / mok::TILE_X;
-    }
-    tab.row_begin[ne] = rows;
-    tab.tile_begin[ne] = tiles;
-  }
+  if (threadIdx.x == 0) tab.fill(g.tokens_per_expert, ne);
   __syncthreads();
 
   const Schedule sched{g, tab, tab.tile_begin[ne], g.op == MOK_GEMM_FWD_ROUTED_DOWN ? 0 : g.num_col_tiles_gate_up,
