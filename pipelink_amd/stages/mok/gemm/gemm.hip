@@ -628,6 +628,9 @@ __device__ __forceinline__ void mainloop(const MokGemmResidue& g, const MokGemmT
   // steady state, every step issuing: what may be outstanding when step t waits for slot t+1
   constexpr int STEADY_EVEN = DEPTH >= 4 ? (DEPTH - 2) * (W_LOADS + X_LOADS / 2) : 0;            // t even
   constexpr int STEADY_ODD = DEPTH >= 4 ? STEADY_EVEN - X_LOADS / 2 : 0;                         // t odd
+  // (the same counts as the run-time formula the tile's last steps use, far from the contraction's end)
+  static_assert(DEPTH < 4 || loads_younger_than_slot<DEPTH>(101, 99, 1 << 20) == STEADY_EVEN, "steady wait of an even step");
+  static_assert(DEPTH < 4 || loads_younger_than_slot<DEPTH>(102, 100, 1 << 20) == STEADY_ODD, "steady wait of an odd step");
 
   // ---- rest of the prologue (steps -DEPTH and 1-DEPTH were issued by `prefetch`), then slot 0's operands
 #pragma unroll
