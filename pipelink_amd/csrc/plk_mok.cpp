@@ -84,10 +84,9 @@ static int make_workspace(plk_mok_session* s, int64_t words) {
     if (hipDeviceSynchronize() != hipSuccess) return plk_hip_set_error(PLK_E_RESOURCE, "plk_mok: device synchronisation failed");
     uint32_t word = 0;
     int rc = plk_hip_readback(&word, s->workspace + MOK_WS_STATUS * 4, sizeof word, nullptr);
-    if (rc == PLK_OK) {
-      s->carried_status |= word;
-      rc = plk_hip_free(s->workspace);
-    }
+    if (rc == PLK_OK) s->carried_status |= word;
+    const int rc_free = plk_hip_free(s->workspace);  // (freed whether or not its status could be read)
+    if (rc == PLK_OK) rc = rc_free;
     s->workspace = 0;
     s->workspace_words = 0;
     if (rc != PLK_OK) return rc;
