@@ -37,6 +37,8 @@
 #include "../include/mok_device.hpp"
 
 extern "C" __device__ int pipelink_mok_gemm_depth();  // ring slots (2 or 4), bound at link time
+#include "load_counts.hpp"
+
 extern "C" __device__ int pipelink_mok_gemm_head();   // byte offset of the rings' first two buffers + scale buffers in dynamic LDS
 extern "C" __device__ int pipelink_mok_gemm_arena();  // byte offset of the rings' other buffers
 
@@ -476,34 +478,10 @@ __device__ __forceinline__ void issue_step(const Loader& ld, const Rings<DEPTH>&
   }
   if (s < n) issue_w(ld, r, s, wb);
 }
-// tile loads issue_step(u) issues: routed rows, weight rows
-template <int DEPTH>
-__device__ __forceinline__ constexpr int x_loads_in(int u, int n) {
-  const int s = u + DEPTH;
-  const int pair = (u & 1) ? s - 1 : s;
-  if (pair >= n) return 0;
-  return DEPTH >= 4 ? X_LOADS / 2 : ((u & 1) == 0 ? X_LOADS : 0);
-}
-template <int DEPTH>
-__device__ __forceinline__ constexpr int w_loads_in(int u, int n) { return u + DEPTH < n ? W_LOADS : 0; }
-// Tile loads that may still be outstanding when slot `slot` is needed and steps up to `last`
-// have been issued (step t waits for slot t+1 with last = t-1; the prologue waits for slot 0
-// with last = -1).  The slot's weight rows are the last loads of step slot-DEPTH; its routed
-// rows come no later, except that with split pairs groups 2-3 of an even slot are issued at
-// the start of step slot+1-DEPTH.
-template <int DEPTH>
-__device__ __forceinline__ constexpr int loads_younger_than_slot(int slot, int last, int n) {
-  int younger = 0;
-  int first = slot + 1 - DEPTH;  // first step all of whose loads are younger
-  if (DEPTH >= 4 && (slot & 1) == 0) {
-    younger += w_loads_in<DEPTH>(first, n);
-    ++first;
-  }
-  for (int u = first; u <= last; ++u) younger += x_loads_in<DEPTH>(u, n) + w_loads_in<DEPTH>(u, n);
-  return younger;
-}
-
-
+// how many tile loads may be in flight behind a slot: load_counts.hpp
+using counts::loads_younger_than_slot;
+using counts::few_younger;
+static_assert(counts::X_LOADS == X_LOADS && counts::W_LOADS == W_LOADS, "the accounting's loads per step are this loader's");
 // ---- tiles of at most 64 routed rows: a deeper ring ---------------------------------------------------------------
 // Such a tile has a quarter of a full tile's MFMAs and as many steps: it takes as long as its loads take to arrive,
 // and a load that is in flight for three steps' time (the full tile's ring) bounds a step from below by a third of
@@ -512,11 +490,12 @@ __device__ __forceinline__ constexpr int loads_younger_than_slot(int slot, int l
 // epilogue uses the arena), four in the arena.  Wave w loads its 64 weight rows as in the full tile and routed rows
 // 16 w .. 16 w + 15; one slot per step, all of it at once (five loads a wave).  Scale buffers and their loads are the
 // full tile's.  Needs the arena of ring depth 4.
-constexpr int FEW_DEPTH = 7;
+constexpr int FEW_DEPTH = counts::FEW_DEPTH;
 constexpr int FEW_HEAD_SLOTS = 3;
 constexpr int FEW_X_BYTES = SMALL_EXTENT * K_SLOT;        // 4 KB
 constexpr int FEW_SLOT_BYTES = BUF_BYTES + FEW_X_BYTES;   // weight rows, then routed rows
-constexpr int FEW_LOADS = W_LOADS + 1;                    // tile loads of one slot, per wave
+constexpr int FEW_LOADS = counts::FEW_LOADS;              // tile loads of one slot, per wave
+static_assert(FEW_LOADS == W_LOADS + 1, "four groups of weight rows and one of routed rows");
 static_assert(FEW_HEAD_SLOTS * FEW_SLOT_BYTES <= 4 * BUF_BYTES, "the first slots fit where the full tile's first buffers are");
 struct FewRing {
   unsigned char* head;
@@ -539,13 +518,6 @@ __device__ __forceinline__ void issue_few(const Loader& ld, const FewRing& ring,
   const uint32_t wslot = (uint32_t)s * ld.w_slot_pitch;
 #pragma unroll
   for (int i = 0; i < W_GROUPS; ++i) buf16_to_lds(ld.w, ld.wsrc[i], wslot, base + ld.dst + i * 1024);
-}
-// tile loads that may still be outstanding when slot `slot` is needed and steps up to `last` have been issued (step u
-// issues slot u + FEW_DEPTH)
-__device__ __forceinline__ int few_younger(int slot, int last, int n) {
-  int younger = 0;
-  for (int u = slot + 1 - FEW_DEPTH; u <= last; ++u) younger += u + FEW_DEPTH < n ? FEW_LOADS : 0;
-  return younger;
 }
 __device__ __forceinline__ void wait_few(int loads) {  // a multiple of FEW_LOADS, at most (FEW_DEPTH - 1) of them
   switch (__builtin_amdgcn_readfirstlane(loads) / FEW_LOADS) {
